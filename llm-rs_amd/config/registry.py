@@ -10,6 +10,7 @@ from typing import Any, Callable, Dict
 from .llama import ConfigError, LlamaConfig
 from .lilatar import LilatarConfig
 from .tuvodra import TuvodraConfig
+from .vivisun import VivisunConfig
 
 # name -> function(config dict) -> typed config with .model_spec() and .to_dict()
 _ARCHITECTURES: Dict[str, Callable[[Dict[str, Any]], Any]] = {}
@@ -60,3 +61,4 @@ def load_config(path: str):
 register_architecture("LlamaForCausalLM", LlamaConfig.from_dict)
 register_architecture("Tuvodra", TuvodraConfig.from_dict)
 register_architecture("Lilatar", LilatarConfig.from_dict)
+register_architecture("Vivisun", VivisunConfig.from_dict)

@@ -8,7 +8,8 @@ and their norms for the usual arrangements (any of them may be left out where
 the arrangement has no use for it), and under `extra` whatever else an
 arrangement of another shape needs (norms after a part, a second feed-forward),
 each with the family it is built from; a `RunSpec` list says which layer runs
-when, so a layer may run twice or read the cache that another run wrote.
+when, so a layer may run twice or read the cache that another run wrote, and whether
+the token embeddings are added to the stream again before it.
 """
 from __future__ import annotations
 
@@ -44,6 +45,9 @@ class LayerSpec:
 class RunSpec:
     layer: int                      # index into ModelSpec.layers
     cache_of: Optional[int] = None  # index of an earlier run whose cache this run reads
+    # the token table's rows (scaled as at the start) are added to the stream again right before this run: for a stretch
+    # of layers that runs several times and is shown its input anew at the start of every further pass
+    add_embedding: bool = False
 
 
 @dataclass(frozen=True)
@@ -79,6 +83,8 @@ class ModelSpec:
         for i, run in enumerate(self.schedule):
             if not 0 <= run.layer < len(self.layers):
                 raise ValueError(f"schedule[{i}] names layer {run.layer}, model has {len(self.layers)}")
+            if run.add_embedding and self.streams > 1:
+                raise ValueError(f"schedule[{i}] adds the embeddings again, which a stream kept in several copies does not take")
             if run.cache_of is not None:
                 if not 0 <= run.cache_of < i:
                     raise ValueError(f"schedule[{i}] reads the cache of run {run.cache_of}, which does not run before it")

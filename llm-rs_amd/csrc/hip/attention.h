@@ -18,11 +18,14 @@ struct AttnArgs {
     // With a window: the first keep_first positions of a request stay visible to every later query, at their true
     // positions.  Key j is visible to the query at i when j <= i and (i - j < window or j < keep_first).
     int keep_first;
+    // sink[head], or null: the softmax's denominator of every query of the head also holds exp(sink[head]), once: a key
+    // without a value, whose score is this number as it stands (not scaled, not bent, no penalty).
+    const float* sink;
 };
 // Whether a call is the plain one (values as wide as keys, no distance penalty, no soft cap, no kept first keys) that
 // every kernel file takes.
 static inline bool attn_is_plain(const AttnArgs& a) {
-    return a.v_dim == a.head_dim && a.dist_r1 == nullptr && a.softcap <= 0.0f && (a.keep_first <= 0 || a.window <= 0);
+    return a.v_dim == a.head_dim && a.dist_r1 == nullptr && a.softcap <= 0.0f && (a.keep_first <= 0 || a.window <= 0) && a.sink == nullptr;
 }
 // The first key of the window of the query at `pos`, and how many of the first keys lie before it and stay visible.
 __host__ __device__ static inline int attn_window_lo(const AttnArgs& a, int pos) {
@@ -33,6 +36,14 @@ __host__ __device__ static inline int attn_kept_before(const AttnArgs& a, int lo
 }
 
 #if defined(__HIPCC__)
+// What the sink of `head` adds to a softmax's sum l whose terms are exp(s - m) (natural: m is a score) or
+// 2^(s log2 e - m) (base 2: m is a score times log2 e); 0 without a sink.  Added once, where the sum is complete.
+__device__ __forceinline__ float attn_sink_term(const AttnArgs& a, int head, float m) {
+    return a.sink ? expf(a.sink[head] - m) : 0.0f;
+}
+__device__ __forceinline__ float attn_sink_term_base2(const AttnArgs& a, int head, float m2) {
+    return a.sink ? __builtin_amdgcn_exp2f(fmaf(a.sink[head], 1.4426950408889634f, -m2)) : 0.0f;
+}
 // A step's entries bring their tokens as tiles of `per` tokens that never cross an entry; entries with one token
 // bring none when the caller splits those by key range instead.  Which entry holds tile `tile`, and which of that
 // entry's tiles it is: a wave finds out together, 64 entries at a time (a serving step has hundreds of entries,

@@ -163,7 +163,7 @@ __global__ __launch_bounds__(256) void attn_f32_tiles_kernel(const float* __rest
     if (a.keep_first > 0 && t_begin > 0) f32_walk<HD>(qf, kc, vc, table, a, kvh, c, h, pos, lo, 0, min(a.keep_first, t_begin), O, m, l);
     f32_walk<HD>(qf, kc, vc, table, a, kvh, c, h, pos, lo, t_begin, t_end, O, m, l);
     if (!cvalid) return;
-    float inv = 1.0f / l;
+    float inv = 1.0f / (l + attn_sink_term_base2(a, head, m));      // (the sum is complete here: the sink joins it once)
     float* op = out + (size_t)token * a.out_stride + (size_t)head * HD + 4 * h;
 #pragma unroll
     for (int dt = 0; dt < HD / 32; ++dt)

@@ -105,6 +105,7 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
     if (kept > 0) walk_keys<T, VEC>(qs, k_cache, v_cache, table, a, kvh, h, pos, 0, kept, m, l, acc);
     walk_keys<T, VEC>(qs, k_cache, v_cache, table, a, kvh, h, pos, lo, pos + 1, m, l, acc);
     T* orow = out + (size_t)t * a.out_stride + (size_t)h * a.v_dim;
+    l += attn_sink_term(a, h, m);
 #pragma unroll
     for (int i = 0; i < MAX_HEAD_DIM / 64; ++i) {
         int d = lane + 64 * i;
@@ -262,10 +263,11 @@ __global__ __launch_bounds__(64) void attention_generic_group_tokens_kernel(
 #pragma unroll
     for (int g = 0; g < G; ++g) {
         T* orow = out + (size_t)t * a.out_stride + (size_t)(kvh * G + g) * a.v_dim;
+        float lg = l[g] + attn_sink_term(a, kvh * G + g, m[g]);
 #pragma unroll
         for (int i = 0; i < NACC; ++i) {
             int d = lane + 64 * i;
-            if (d < a.v_dim) orow[d] = from_f32<T>(acc[g][i] / l[g]);
+            if (d < a.v_dim) orow[d] = from_f32<T>(acc[g][i] / lg);
         }
     }
 }
@@ -364,6 +366,7 @@ __global__ __launch_bounds__(64) void attention_generic_merge_kernel(
         }
     }
     T* orow = out + (size_t)t * a.out_stride + (size_t)h * hd;
+    L += attn_sink_term(a, h, M);
 #pragma unroll
     for (int i = 0; i < MAX_HEAD_DIM / 64; ++i) {
         int d = lane + 64 * i;
@@ -475,6 +478,7 @@ static int launch_generic(hipStream_t stream, const T* q, T* out, const T* k_cac
 // v_dim: the width of a value (the cache's values are [page][kv_head][v_dim][slot], `out` has v_dim per head);
 // dist_r1, dist_r2: [n_heads] 32-bit, the logarithmic distance penalty of AttnArgs, or both null.
 // softcap, keep_first: the soft cap of the scores and the first keys that a window keeps (AttnArgs), or 0.
+// sink: [n_heads] 32-bit, a number a head that the softmax's denominator also holds the exponential of, or null.
 extern "C" int llmrs_attention_ext(hipStream_t stream, int dtype, const void* q, int q_stride, void* out, int out_stride,
                                    const void* k_cache, const void* v_cache, const int* block_table, int table_width,
                                    const int* token_entry, const int* positions, const int* q_starts,
@@ -482,7 +486,7 @@ extern "C" int llmrs_attention_ext(hipStream_t stream, int dtype, const void* q,
                                    int head_dim, int page_size, int num_pages, int window, float scale,
                                    void* scratch, size_t scratch_bytes, int max_seq_len, int n_single, long single_keys,
                                    int allow_mfma, int v_dim, const float* dist_r1, const float* dist_r2, float softcap,
-                                   int keep_first) {
+                                   int keep_first, const float* sink) {
     LLMRS_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && head_dim > 0 && v_dim > 0, "attention: bad sizes");
     LLMRS_REQUIRE(v_dim <= MAX_HEAD_DIM, "attention: value width %d exceeds %d", v_dim, MAX_HEAD_DIM);
     LLMRS_REQUIRE((dist_r1 == nullptr) == (dist_r2 == nullptr), "attention: the distance penalty needs both of its tables");
@@ -498,7 +502,7 @@ extern "C" int llmrs_attention_ext(hipStream_t stream, int dtype, const void* q,
                   "attention: every entry is said to bring one token, but %d entries bring %d tokens", n_entries, n_tokens);
     if (n_tokens == 0) return 0;
     AttnArgs a{n_tokens, n_heads, n_kv_heads, head_dim, page_size, table_width, num_pages, q_stride, out_stride, window, scale,
-               v_dim, dist_r1, dist_r2, softcap, window > 0 ? keep_first : 0};
+               v_dim, dist_r1, dist_r2, softcap, window > 0 ? keep_first : 0, sink};
     if (dtype == LLMRS_BF16 && allow_mfma) {
         int took = llmrs_attention_bf16_mfma(stream, (const bf16*)q, (bf16*)out, (const bf16*)k_cache, (const bf16*)v_cache,
                                              block_table, token_entry, positions, q_starts, seq_lens, n_entries,
@@ -531,5 +535,5 @@ extern "C" int llmrs_attention(hipStream_t stream, int dtype, const void* q, int
     return llmrs_attention_ext(stream, dtype, q, q_stride, out, out_stride, k_cache, v_cache, block_table, table_width,
                                token_entry, positions, q_starts, seq_lens, n_entries, n_tokens, n_heads, n_kv_heads,
                                head_dim, page_size, num_pages, window, scale, scratch, scratch_bytes, max_seq_len, n_single,
-                               single_keys, allow_mfma, head_dim, nullptr, nullptr, 0.0f, 0);
+                               single_keys, allow_mfma, head_dim, nullptr, nullptr, 0.0f, 0, nullptr);
 }

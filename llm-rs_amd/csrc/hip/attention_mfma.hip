@@ -287,7 +287,7 @@ __global__ __launch_bounds__(256) void attn_tiles_kernel(const bf16* __restrict_
                      a.n_kv_heads, kvh, t_begin, t_end, pos, lo, a.scale, false, 0,
                      a.dist_r1 != nullptr, a.dist_r1 ? a.dist_r1[head] : 0.0f, a.dist_r1 ? a.dist_r2[head] : 0.0f, bend);
     if (!cvalid) return;
-    float inv = 1.0f / l;
+    float inv = 1.0f / (l + attn_sink_term_base2(a, head, m));      // (the sum is complete here: the sink joins it once)
     bf16* op = out + (size_t)token * a.out_stride + (size_t)head * HD;
 #pragma unroll
     for (int dt = 0; dt < HD / 32; ++dt)
@@ -552,7 +552,7 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(HD <
     }
 
     if (!cvalid) return;
-    float inv = 1.0f / l;
+    float inv = 1.0f / (l + attn_sink_term_base2(a, head, m));      // (the sum is complete here: the sink joins it once)
     bf16* op = out + (size_t)token * a.out_stride + (size_t)head * HD;
 #pragma unroll
     for (int dt = 0; dt < HD / 32; ++dt)
@@ -923,7 +923,7 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(const float* __restrict
         for (int c = 0; c < AHEAD; ++c)
             if (ch + c < n_chunks) o = fmaf(v[c], weight[ch + c], o);
     }
-    out[(size_t)token * a.out_stride + (size_t)head * hd + d] = (bf16)(o / L);
+    out[(size_t)token * a.out_stride + (size_t)head * hd + d] = (bf16)(o / (L + attn_sink_term_base2(a, head, M)));
 }
 
 // The merge for more than a few chunks (131,000 keys of one request are 256 chunks of 512).  One thread per
@@ -1005,7 +1005,7 @@ __global__ __launch_bounds__(MERGE_GROUP_THREADS) void attn_merge_groups_kernel(
     if (tid < hd) {
         float o = 0.0f;
         for (int k = 0; k < groups; ++k) o += sums[k * hd + tid];
-        out[(size_t)token * a.out_stride + (size_t)head * hd + tid] = (bf16)(o / L);
+        out[(size_t)token * a.out_stride + (size_t)head * hd + tid] = (bf16)(o / (L + attn_sink_term_base2(a, head, M)));
     }
 }
 

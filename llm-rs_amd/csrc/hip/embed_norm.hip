@@ -21,7 +21,8 @@ __device__ __forceinline__ bool rows_by_eights(const T* table, const float* out,
 
 // out[t, :] = float(table[tokens[t], :]) * scale   (reference: embed_batch_*, shaders/ops.metal:878-915,
 // which has no scale: 1 there and for every architecture that does not ask for one)
-template <class T>
+// ADD: out[t, :] += the same, in 32-bit (a stream that is shown its tokens' embeddings again).
+template <class T, bool ADD>
 __global__ void embed_rows_kernel(float* __restrict__ out, const T* __restrict__ table,
                                   const int* __restrict__ tokens, int D, int V, float scale) {
     int t = blockIdx.x;
@@ -34,12 +35,17 @@ __global__ void embed_rows_kernel(float* __restrict__ out, const T* __restrict__
             for (int d = threadIdx.x * 8; d < D; d += blockDim.x * 8) {
                 float v[8];
                 load8_scaled((const bf16*)src + d, scale, v);
+                if constexpr (ADD) {
+                    embed_f32x4 a = *(const embed_f32x4*)(dst + d), b = *(const embed_f32x4*)(dst + d + 4);
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) { v[j] += a[j]; v[4 + j] += b[j]; }
+                }
                 store8(dst + d, v);
             }
             return;
         }
     }
-    for (int d = threadIdx.x; d < D; d += blockDim.x) dst[d] = to_f32(src[d]) * scale;
+    for (int d = threadIdx.x; d < D; d += blockDim.x) dst[d] = (ADD ? dst[d] : 0.0f) + to_f32(src[d]) * scale;
 }
 
 // One block per row: ss = sum x^2 in 32-bit, inv = 1/sqrt(ss/D + eps),
@@ -121,18 +127,27 @@ __global__ void rmsnorm_rows_reg_kernel(T* __restrict__ out, const float* __rest
     }
 }
 
-extern "C" int llmrs_embed_rows(hipStream_t stream, int dtype, float* out, const void* table, const int* tokens,
-                                int n_tokens, int D, int V, float scale) {
+template <bool ADD>
+static int embed_rows(hipStream_t stream, int dtype, float* out, const void* table, const int* tokens, int n_tokens, int D, int V, float scale) {
     LLMRS_REQUIRE(n_tokens >= 0 && D > 0 && V > 0, "embed_rows: bad sizes T=%d D=%d V=%d", n_tokens, D, V);
     if (n_tokens == 0) return 0;
     if (dtype == LLMRS_F32)
-        embed_rows_kernel<float><<<n_tokens, 256, 0, stream>>>(out, (const float*)table, tokens, D, V, scale);
+        embed_rows_kernel<float, ADD><<<n_tokens, 256, 0, stream>>>(out, (const float*)table, tokens, D, V, scale);
     else if (dtype == LLMRS_BF16)
-        embed_rows_kernel<bf16><<<n_tokens, 256, 0, stream>>>(out, (const bf16*)table, tokens, D, V, scale);
+        embed_rows_kernel<bf16, ADD><<<n_tokens, 256, 0, stream>>>(out, (const bf16*)table, tokens, D, V, scale);
     else
         return llmrs_fail("embed_rows: unknown dtype %d", dtype);
     LLMRS_LAUNCH_CHECK("embed_rows");
     return 0;
+}
+extern "C" int llmrs_embed_rows(hipStream_t stream, int dtype, float* out, const void* table, const int* tokens,
+                                int n_tokens, int D, int V, float scale) {
+    return embed_rows<false>(stream, dtype, out, table, tokens, n_tokens, D, V, scale);
+}
+// out[t, :] += float(table[tokens[t], :]) * scale
+extern "C" int llmrs_embed_rows_add(hipStream_t stream, int dtype, float* out, const void* table, const int* tokens,
+                                    int n_tokens, int D, int V, float scale) {
+    return embed_rows<true>(stream, dtype, out, table, tokens, n_tokens, D, V, scale);
 }
 
 // rows == nullptr: row i of x -> row i of out; else row rows[i] of x -> row i of out.

@@ -1,0 +1,133 @@
+// Kernels of latent attention: keys and values of all heads are matrices times one small vector c per token, and only
+// c is cached.  Attention then runs in the latent space (attention*.hip, one key head of width `rank` whose values are
+// its keys), between two products that carry every head's query into that space and its result out of it.
+//
+//   latent_finish: the input product's 32-bit sums -> q in the activation type; c = rmsnorm(sums_c) * weight into its
+//                  page twice: as a row of the keys [page][slot][rank], as a column of the values [page][rank][slot]
+//   head_product:  out[t, h, :] = W[h] a[t, h, :], every head by its own small matrix, optionally times
+//                  sigmoid(gate[t, h]) computed on the 32-bit sums
+#include "cache_layout.h"
+#include "common.h"
+#include "gemm.h"
+
+template <class T>
+__global__ __launch_bounds__(256) void latent_finish_kernel(const float* __restrict__ sums, int ld, T* __restrict__ q, int ldq,
+                                                            int q_size, int rank, const float* __restrict__ weight, float eps,
+                                                            const int* __restrict__ slot_map, T* __restrict__ k_cache,
+                                                            T* __restrict__ v_cache, int page_size, int num_pages, int write) {
+    int t = blockIdx.x;
+    const float* src = sums + (size_t)t * ld;
+    for (int d = threadIdx.x; d < q_size; d += 256) q[(size_t)t * ldq + d] = from_f32<T>(src[d]);
+    if (threadIdx.x >= 64 || !write) return;
+    int lane = threadIdx.x;
+    float x[8];            // features lane, lane + 64, ... (up to 512)
+    float ss = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        int d = lane + 64 * i;
+        x[i] = d < rank ? src[q_size + d] : 0.0f;
+        ss = fmaf(x[i], x[i], ss);
+    }
+    float inv = 1.0f / sqrtf(wave_sum(ss) / (float)rank + eps);
+    int slot = slot_map[t];
+    if (slot < 0 || slot >= num_pages * page_size) return;  // never write outside the cache
+    int page = slot / page_size, off = slot % page_size;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        int d = lane + 64 * i;
+        if (d >= rank) continue;
+        T c = from_f32<T>(x[i] * inv * weight[d]);
+        k_cache[k_cache_index(page, 0, off, d, 1, page_size, rank)] = c;
+        v_cache[v_cache_index(page, 0, off, d, 1, page_size, rank)] = c;
+    }
+}
+
+// sums: [n_tokens, ld] 32-bit, a token's q (q_size columns), then its c (rank columns); q: [n_tokens, ldq] in `dtype`;
+// weight: [rank] 32-bit; the caches in `dtype`; slot_map: [n_tokens] page * page_size + slot.
+extern "C" int llmrs_latent_finish(hipStream_t stream, int dtype, const float* sums, int ld, void* q, int ldq, int n_tokens,
+                                   int q_size, int rank, const float* weight, float eps, const int* slot_map, void* k_cache,
+                                   void* v_cache, int page_size, int num_pages, int write) {
+    LLMRS_REQUIRE(n_tokens >= 0 && q_size > 0 && rank > 0 && ld >= q_size + rank && ldq >= q_size, "latent_finish: bad sizes");
+    LLMRS_REQUIRE(rank <= 512, "latent_finish: a latent vector of %d numbers exceeds 512", rank);
+    LLMRS_REQUIRE(eps > 0.0f && weight, "latent_finish: the norm needs its weight and a positive eps");
+    LLMRS_REQUIRE(!write || (page_size > 0 && num_pages > 0 && slot_map && k_cache && v_cache), "latent_finish: no cache to write");
+    if (n_tokens == 0) return 0;
+    if (dtype == LLMRS_F32)
+        latent_finish_kernel<float><<<n_tokens, 256, 0, stream>>>(sums, ld, (float*)q, ldq, q_size, rank, weight, eps, slot_map,
+                                                                   (float*)k_cache, (float*)v_cache, page_size, num_pages, write);
+    else if (dtype == LLMRS_BF16)
+        latent_finish_kernel<bf16><<<n_tokens, 256, 0, stream>>>(sums, ld, (bf16*)q, ldq, q_size, rank, weight, eps, slot_map,
+                                                                  (bf16*)k_cache, (bf16*)v_cache, page_size, num_pages, write);
+    else
+        return llmrs_fail("latent_finish: unknown dtype %d", dtype);
+    LLMRS_LAUNCH_CHECK("latent_finish");
+    return 0;
+}
+
+// ---- every head by its own matrix -----------------------------------------------------------------------------------
+// A block of 256 threads makes 64 tokens x 64 outputs of one head: 16 inputs at a time through LDS, every thread a
+// 4 x 4 corner in 32-bit multiply-adds (any sizes, any type).
+#define HP_TILE 64
+#define HP_K 16
+template <class T>
+__global__ __launch_bounds__(256) void head_product_kernel(const T* __restrict__ a, int lda, const T* __restrict__ w,
+                                                           T* __restrict__ out, int ldo, int n_tokens, int n_in, int n_out,
+                                                           const float* __restrict__ gate, int ldg) {
+    __shared__ float As[HP_K][HP_TILE + 4], Ws[HP_K][HP_TILE + 4];
+    int h = blockIdx.z, m0 = blockIdx.y * HP_TILE, n0 = blockIdx.x * HP_TILE, tid = threadIdx.x;
+    const T* ah = a + (size_t)h * n_in;
+    const T* wh = w + (size_t)h * n_out * n_in;
+    int tm = (tid >> 4) * 4, tn = (tid & 15) * 4;
+    int lr = tid >> 2, lk = (tid & 3) * 4;          // this thread's share of a tile's loads: row lr, inputs lk .. lk + 3
+    float acc[4][4] = {};
+    for (int k0 = 0; k0 < n_in; k0 += HP_K) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            int k = k0 + lk + j;
+            As[lk + j][lr] = (m0 + lr < n_tokens && k < n_in) ? to_f32(ah[(size_t)(m0 + lr) * lda + k]) : 0.0f;
+            Ws[lk + j][lr] = (n0 + lr < n_out && k < n_in) ? to_f32(wh[(size_t)(n0 + lr) * n_in + k]) : 0.0f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < HP_K; ++k) {
+            float av[4], wv[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { av[i] = As[k][tm + i]; wv[i] = Ws[k][tn + i]; }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(av[i], wv[j], acc[i][j]);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        int m = m0 + tm + i;
+        if (m >= n_tokens) continue;
+        float g = gate ? 1.0f / (1.0f + expf(-gate[(size_t)m * ldg + h])) : 1.0f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            int n = n0 + tn + j;
+            if (n < n_out) out[(size_t)m * ldo + (size_t)h * n_out + n] = from_f32<T>(acc[i][j] * g);
+        }
+    }
+}
+
+// a: [n_tokens, lda], head h's inputs at columns h * n_in ..; w: [heads][n_out][n_in]; out: [n_tokens, ldo], head h's
+// outputs at columns h * n_out ..; all in `dtype`, sums in 32-bit.  gate: [n_tokens, ldg] 32-bit, a column a head, or null.
+extern "C" int llmrs_head_product(hipStream_t stream, int dtype, const void* a, int lda, const void* w, void* out, int ldo,
+                                  int n_tokens, int heads, int n_in, int n_out, int allow_mfma, const float* gate, int ldg) {
+    LLMRS_REQUIRE(n_tokens >= 0 && heads > 0 && n_in > 0 && n_out > 0, "head_product: bad sizes");
+    LLMRS_REQUIRE(lda >= heads * n_in && ldo >= heads * n_out && (gate == nullptr || ldg >= heads), "head_product: row stride too short");
+    LLMRS_REQUIRE(heads <= 65535 && ceil_div(n_tokens, HP_TILE) <= 65535, "head_product: too many heads or tokens for one launch");
+    LLMRS_REQUIRE(dtype == LLMRS_F32 || dtype == LLMRS_BF16, "head_product: unknown dtype %d", dtype);
+    if (n_tokens == 0) return 0;
+    (void)allow_mfma;
+    dim3 grid(ceil_div(n_out, HP_TILE), ceil_div(n_tokens, HP_TILE), heads);
+    if (dtype == LLMRS_F32)
+        head_product_kernel<float><<<grid, 256, 0, stream>>>((const float*)a, lda, (const float*)w, (float*)out, ldo, n_tokens, n_in, n_out, gate, ldg);
+    else
+        head_product_kernel<bf16><<<grid, 256, 0, stream>>>((const bf16*)a, lda, (const bf16*)w, (bf16*)out, ldo, n_tokens, n_in, n_out, gate, ldg);
+    LLMRS_LAUNCH_CHECK("head_product");
+    return 0;
+}

@@ -1,10 +1,14 @@
 // What lies between a q/k/v projection and attention for mixers that do more to q and k than rotate them:
-// biases, a norm of q and k to unit root mean square per head, a rotation by position, and the write of k and v into
-// the paged cache, in one pass over the projection's 32-bit sums.
+// a short causal convolution over time, biases, a norm of q and k to unit root mean square per head (with or without a
+// weight), a rotation by position, and the write of k and v into the paged cache, in one pass over the projection's
+// 32-bit sums.
 //
-//   q[t, h, :] = rot(unit(sums_q[t, h, :] + bias_q[h, :]))   unit(x) = x / sqrt(mean(x^2) + eps) over the head (eps 0: x)
-//   rot: features (2i, 2i + 1), i < rotary_dim / 2, turned by the angle position * inv_freq[i]; the others pass
-//   k likewise, into its page; v[t, g, :] = sums_v + bias_v, into its page (values lie transposed, cache_layout.h).
+//   u[t, c] = sum_j taps[c, j] * sums[t - (K - 1 - j), c]     (with taps; rows before an entry's first token come from
+//             the request's state, [K - 1][columns] 32-bit, whose last row is the token before the entry)
+//   q[t, h, :] = rot(unit(u_q[t, h, :] + bias_q[h, :]) * w_q)   unit(x) = x / sqrt(mean(x^2) + eps) over the head (eps 0: x)
+//   rot: features (2i, 2i + 1), i < rotary_dim / 2, turned by the angle position * inv_freq[i], cosine and sine both
+//        times `gain`; the others pass
+//   k likewise (weight w_k), into its page; v[t, g, :] = u_v + bias_v, into its page (values lie transposed, cache_layout.h).
 // Everything is computed in 32-bit and rounded once to the activation type on the way out.
 #include "cache_layout.h"
 #include "common.h"
@@ -15,6 +19,17 @@ struct QkvFinishArgs {
     int page_size, num_pages, write_kv;
     float eps;                     // of the unit norm; 0: q and k are not normed
     int rotary_dim;                // 0: no rotation
+    float gain;                    // cosine and sine are multiplied by this
+    const float* q_weight;         // [head_dim] each, or null: what the normed q and k are multiplied by
+    const float* k_weight;
+    // the convolution (taps null: none): taps [columns][n_taps]; state [slots][n_taps - 1][columns] at state_stride a slot
+    const float* taps;
+    int n_taps, columns;
+    const float* state;
+    long state_stride;
+    const int* q_starts;
+    const int* slots;
+    const int* token_entry;
 };
 
 // One wave for each (token, head of q, k or v).
@@ -34,14 +49,47 @@ __global__ __launch_bounds__(64) void qkv_finish_kernel(const float* __restrict_
     const float* src = sums + (size_t)t * a.in_stride + col;
     float x[8];            // features lane, lane + 64, ... (heads of up to 512)
     float ss = 0.0f;
+    if (a.taps) {
+        int e = a.token_entry[t];
+        int place = t - a.q_starts[e];                     // the token's place in its entry
+        const float* sp = a.n_taps > 1 ? a.state + (size_t)a.slots[e] * a.state_stride + col : nullptr;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        int d = lane + 64 * i;
-        x[i] = d < width ? src[d] + (bias ? bias[col + d] : 0.0f) : 0.0f;
-        ss = fmaf(x[i], x[i], ss);
+        for (int i = 0; i < 8; ++i) {
+            int d = lane + 64 * i;
+            float acc = 0.0f;
+            if (d < width) {
+                const float* w = a.taps + (size_t)(col + d) * a.n_taps;
+                for (int j = 0; j < a.n_taps; ++j) {
+                    int back = a.n_taps - 1 - j;           // how many tokens before this one
+                    float in = place - back >= 0 ? src[d - (long)back * a.in_stride]
+                                                 : sp[(size_t)(a.n_taps - 1 + place - back) * a.columns + d];
+                    acc = fmaf(w[j], in, acc);
+                }
+            }
+            x[i] = acc;
+            ss = fmaf(acc, acc, ss);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            int d = lane + 64 * i;
+            x[i] = d < width ? src[d] + (bias ? bias[col + d] : 0.0f) : 0.0f;
+            ss = fmaf(x[i], x[i], ss);
+        }
     }
     float inv = 1.0f;
-    if ((is_q || is_k) && a.eps > 0.0f) inv = 1.0f / sqrtf(wave_sum(ss) / (float)width + a.eps);
+    if ((is_q || is_k) && a.eps > 0.0f) {
+        inv = 1.0f / sqrtf(wave_sum(ss) / (float)width + a.eps);
+        const float* nw = is_q ? a.q_weight : a.k_weight;
+        if (nw) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                int d = lane + 64 * i;
+                x[i] = d < width ? x[i] * inv * nw[d] : 0.0f;
+            }
+            inv = 1.0f;
+        }
+    }
     if ((is_q || is_k) && a.rotary_dim > 0) {
         // feature d's partner d ^ 1 lies in the neighbouring lane; angles and the turn in 32-bit
         float pos = (float)positions[t];
@@ -53,6 +101,8 @@ __global__ __launch_bounds__(64) void qkv_finish_kernel(const float* __restrict_
             if (d < a.rotary_dim) {
                 float s, c;
                 sincosf(pos * inv_freq[d >> 1], &s, &c);
+                s *= a.gain;
+                c *= a.gain;
                 x[i] = (d & 1) ? fmaf(x[i], c, other * s) : fmaf(x[i], c, -other * s);
             }
         }
@@ -84,11 +134,16 @@ __global__ __launch_bounds__(64) void qkv_finish_kernel(const float* __restrict_
 // sums: [n_tokens, in_stride] 32-bit, a token's q heads, then its k heads, then its v heads; bias: the same columns
 // (or null); q: [n_tokens, q_stride] in `dtype`; the caches in `dtype`; slot_map: [n_tokens] page * page_size + slot.
 // n_kv_heads 0: the projection has no k and v (a mixer that reads another's cache).
-// positions: [n_tokens], inv_freq: [rotary_dim / 2] 32-bit, for the rotation (rotary_dim 0: none).
+// positions: [n_tokens], inv_freq: [rotary_dim / 2] 32-bit, for the rotation (rotary_dim 0: none); gain: see above.
+// q_weight, k_weight: [head_dim] 32-bit or null.  taps: [columns of q | k | v][n_taps] 32-bit or null; then state (null when
+// n_taps == 1), q_starts [n_entries + 1], slots [n_entries], token_entry [n_tokens] say where a token's earlier rows lie.
+// The state is only read here: llmrs_conv_state_update brings it up to date afterwards.
 extern "C" int llmrs_qkv_finish(hipStream_t stream, int dtype, const float* sums, int in_stride, const float* bias, void* q,
                                 int q_stride, const int* slot_map, void* k_cache, void* v_cache, int n_tokens, int n_heads,
                                 int n_kv_heads, int head_dim, int v_dim, int page_size, int num_pages, int write_kv, float eps,
-                                const int* positions, const float* inv_freq, int rotary_dim) {
+                                const int* positions, const float* inv_freq, int rotary_dim, const float* q_weight,
+                                const float* k_weight, float gain, const float* taps, int n_taps, const float* state,
+                                long state_stride, const int* q_starts, const int* slots, const int* token_entry, int n_entries) {
     LLMRS_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv_heads >= 0 && head_dim > 0 && v_dim > 0, "qkv_finish: bad sizes");
     LLMRS_REQUIRE(head_dim <= 512 && v_dim <= 512, "qkv_finish: heads of %d / %d features exceed 512", head_dim, v_dim);
     LLMRS_REQUIRE(in_stride >= (n_heads + n_kv_heads) * head_dim + n_kv_heads * v_dim && q_stride >= n_heads * head_dim,
@@ -98,8 +153,16 @@ extern "C" int llmrs_qkv_finish(hipStream_t stream, int dtype, const float* sums
     LLMRS_REQUIRE(rotary_dim == 0 || (positions && inv_freq), "qkv_finish: a rotation needs positions and frequencies");
     LLMRS_REQUIRE(!write_kv || (page_size > 0 && num_pages > 0 && slot_map && k_cache && v_cache), "qkv_finish: no cache to write");
     LLMRS_REQUIRE(n_heads + 2 * n_kv_heads <= 65535, "qkv_finish: too many heads for one launch");
+    LLMRS_REQUIRE((q_weight == nullptr && k_weight == nullptr) || eps > 0.0f, "qkv_finish: a norm's weight without the norm");
+    int columns = (n_heads + n_kv_heads) * head_dim + n_kv_heads * v_dim;
+    if (taps) {
+        LLMRS_REQUIRE(n_taps >= 1 && bias == nullptr, "qkv_finish: a convolution needs at least one tap and goes without biases");
+        LLMRS_REQUIRE(q_starts && slots && token_entry && n_entries > 0, "qkv_finish: a convolution needs the step's entries");
+        LLMRS_REQUIRE(n_taps == 1 || (state && state_stride >= (long)(n_taps - 1) * columns), "qkv_finish: the convolution's state is too small");
+    }
     if (n_tokens == 0) return 0;
-    QkvFinishArgs a{n_tokens, n_heads, n_kv_heads, head_dim, v_dim, in_stride, q_stride, page_size, num_pages, write_kv, eps, rotary_dim};
+    QkvFinishArgs a{n_tokens, n_heads, n_kv_heads, head_dim, v_dim, in_stride, q_stride, page_size, num_pages, write_kv, eps, rotary_dim,
+                    gain, q_weight, k_weight, taps, n_taps, columns, state, state_stride, q_starts, slots, token_entry};
     dim3 grid(n_tokens, n_heads + 2 * n_kv_heads);
     if (dtype == LLMRS_F32)
         qkv_finish_kernel<float><<<grid, 64, 0, stream>>>(sums, bias, (float*)q, slot_map, (float*)k_cache, (float*)v_cache, positions, inv_freq, a);

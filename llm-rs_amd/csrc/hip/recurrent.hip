@@ -384,6 +384,18 @@ extern "C" int llmrs_causal_conv_silu(hipStream_t stream, int dtype, const float
     return 0;
 }
 
+// The state of a causal convolution alone (for a caller that convolves in a kernel of its own): the last K - 1 rows of
+// (old state, this step's rows of sums) for every entry.  Launch it after whatever still reads the old state.
+extern "C" int llmrs_conv_state_update(hipStream_t stream, const float* sums, int ld, float* state, long state_stride,
+                                       const int* q_starts, const int* slots, int n_entries, int C, int K) {
+    LLMRS_REQUIRE(C > 0 && K >= 1 && ld >= C && state_stride >= (long)(K - 1) * C, "conv_state_update: bad sizes");
+    LLMRS_REQUIRE(entries_ok(q_starts, slots, n_entries) && n_entries <= 65535, "conv_state_update: bad entries");
+    if (K == 1 || n_entries == 0) return 0;
+    causal_conv_state_kernel<<<dim3(ceil_div(C, 64), n_entries), 64, 0, stream>>>(sums, ld, state, state_stride, q_starts, slots, C, K);
+    LLMRS_LAUNCH_CHECK("conv_state_update");
+    return 0;
+}
+
 // x: [T, ldx] the convolution's output; bc: [T, ldbc] with B at column off_b and C at off_c, N wide each; both and
 // `out` in `dtype`.  ypart: [T, C] 32-bit, needed only when N > 64.  longest: the most tokens any entry brings (an
 // upper bound will do).  carry: [llmrs_scan_places][N + 1][C] floats, or null; with it, entries longer than a chunk

@@ -92,3 +92,29 @@ extern "C" int llmrs_add_bias_rows(hipStream_t stream, float* rows, int ld, cons
     LLMRS_LAUNCH_CHECK("add_bias_rows");
     return 0;
 }
+
+// o[t, j] *= sigmoid(gate[t, j / per]) in place: an output gate on a mixer's heads, one gate for every feature (per 1)
+// or one for each group of `per` features (a head).  The gate is a product's 32-bit sums; sigmoid and product are 32-bit.
+template <class T>
+__global__ void sigmoid_gate_kernel(T* __restrict__ o, int ldo, const float* __restrict__ gate, int ldg, int n, int per, long total) {
+    long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    long t = i / n;
+    int c = (int)(i - t * n);
+    float g = gate[(size_t)t * ldg + c / per];
+    T* p = o + (size_t)t * ldo + c;
+    *p = from_f32<T>(to_f32(*p) / (1.0f + expf(-g)));
+}
+
+extern "C" int llmrs_sigmoid_gate(hipStream_t stream, int dtype, void* o, int ldo, const float* gate, int ldg, int n_rows, int n, int per) {
+    LLMRS_REQUIRE(o && gate && n > 0 && per > 0 && n % per == 0 && ldo >= n && ldg >= n / per && n_rows >= 0, "sigmoid_gate: bad arguments");
+    long total = (long)n_rows * n;
+    if (total == 0) return 0;
+    LLMRS_REQUIRE((total + 255) / 256 <= 0x7fffffffL, "sigmoid_gate: too many elements for one launch");
+    int blocks = (int)((total + 255) / 256);
+    if (dtype == LLMRS_F32) sigmoid_gate_kernel<float><<<blocks, 256, 0, stream>>>((float*)o, ldo, gate, ldg, n, per, total);
+    else if (dtype == LLMRS_BF16) sigmoid_gate_kernel<bf16><<<blocks, 256, 0, stream>>>((bf16*)o, ldo, gate, ldg, n, per, total);
+    else return llmrs_fail("sigmoid_gate: unknown dtype %d", dtype);
+    LLMRS_LAUNCH_CHECK("sigmoid_gate");
+    return 0;
+}

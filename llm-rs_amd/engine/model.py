@@ -129,8 +129,13 @@ class Model:
             # the norm that reads the stream after this block: the next block's first; after the last block the
             # final norm, where it reads every row (else it reads gathered rows and runs as a kernel of its own)
             later = self.spec.schedule[i + 1] if i + 1 < len(self.spec.schedule) else None
-            ctx.norm_after_block = (self.blocks[later.layer].first_norm() if later is not None
+            # (a run that adds the embeddings first changes the stream before its norm reads it: nothing to prepare)
+            ctx.norm_after_block = (None if later is not None and later.add_embedding
+                                    else self.blocks[later.layer].first_norm() if later is not None
                                     else self.final_norm if ctx.wants_every_row else None)      # (None too without a final norm)
+            if run.add_embedding:          # the tokens' embeddings once more, as they entered the stream at the start
+                k.embed_rows(h, self.embedding, ctx.tokens, self.spec.embedding_scale, add=True)
+                ctx.note_left(h, None)
             block.forward(ctx, h, cache_views[i])
             if not block.keeps_left_current:
                 ctx.note_left(h, None)

@@ -174,6 +174,12 @@ class HipKernels(Kernels):
         V, I, F = c_void_p, c_int, c_float
         sigs = {
             "llmrs_embed_rows": [V, I, V, V, V, I, I, I, F],
+            "llmrs_embed_rows_add": [V, I, V, V, V, I, I, I, F],
+            "llmrs_dyt": [V, I, V, V, V, V, V, V, I, I, V, V, V, V],
+            "llmrs_conv_state_update": [V, V, I, V, ctypes.c_long, V, V, I, I, I],
+            "llmrs_sigmoid_gate": [V, I, V, I, V, I, I, I, I],
+            "llmrs_latent_finish": [V, I, V, I, V, I, I, I, I, V, F, V, V, V, I, I, I],
+            "llmrs_head_product": [V, I, V, I, V, V, I, I, I, I, I, I, V, I],
             "llmrs_fill_normal": [V, I, V, c_size_t, ctypes.c_uint64, ctypes.c_uint64, F, F],
             "llmrs_cast": [V, V, I, V, I, c_size_t],
             "llmrs_scale_softcap_rows": [V, V, I, I, I, F, F],
@@ -188,11 +194,11 @@ class HipKernels(Kernels):
             "llmrs_argmax_rows": [V, V, I, I, I, V, V, c_size_t],
             "llmrs_sample_rows": [V, V, I, I, I, V, V],
             "llmrs_place_ids": [V, V, I, V, V, V, I, I, I],
-            "llmrs_attention_ext": [V, I, V, I, V, I, V, V, V, I, V, V, V, V, I, I, I, I, I, I, I, I, F, V, c_size_t, I, I, ctypes.c_long, I, I, V, V, F, I],
+            "llmrs_attention_ext": [V, I, V, I, V, I, V, V, V, I, V, V, V, V, I, I, I, I, I, I, I, I, F, V, c_size_t, I, I, ctypes.c_long, I, I, V, V, F, I, V],
             "llmrs_group_rmsnorm": [V, I, V, V, ctypes.c_long, I, V, V, V, I, I, I, F, V, V, V, V, V],
             "llmrs_streams_mix": [V, V, ctypes.c_long, I, V, V, V, ctypes.c_long],
             "llmrs_streams_copy_first": [V, V, ctypes.c_long, I, ctypes.c_long],
-            "llmrs_qkv_finish": [V, I, V, I, V, V, I, V, V, V, I, I, I, I, I, I, I, I, F, V, V, I],
+            "llmrs_qkv_finish": [V, I, V, I, V, V, I, V, V, V, I, I, I, I, I, I, I, I, F, V, V, I, V, V, F, V, I, V, ctypes.c_long, V, V, V, I],
             "llmrs_linear_scan": [V, V, I, V, I, V, I, V, I, V, V, I, V, ctypes.c_long, V, V, I, I, I, I, I, I, V, I],
             "llmrs_silu_columns": [V, V, I, I, I, I],
             "llmrs_delta_prepare": [V, V, I, V, I, V, I, V, I, V, V, I, I, I, I, F],
@@ -297,11 +303,12 @@ class HipKernels(Kernels):
         return torch.cuda.current_stream().cuda_stream
 
     # out[t, :] = table[tokens[t], :] * scale as float32
-    def embed_rows(self, out: torch.Tensor, table: torch.Tensor, tokens: torch.Tensor, scale: float = 1.0) -> None:
+    # (add: out[t, :] += the same, for a stream that is shown its tokens' embeddings again)
+    def embed_rows(self, out: torch.Tensor, table: torch.Tensor, tokens: torch.Tensor, scale: float = 1.0, add: bool = False) -> None:
         assert out.dtype == torch.float32 and tokens.dtype == torch.int32 and table.is_contiguous() and out.is_contiguous()
         assert out.shape[0] == tokens.shape[0] and out.shape[1] == table.shape[1]
-        self._run("embed", out.numel() * (4 + table.element_size()), 0, None,
-                  self.lib.llmrs_embed_rows, self._stream(), _code(table.dtype), _p(out), _p(table), _p(tokens),
+        self._run("embed add" if add else "embed", out.numel() * ((8 if add else 4) + table.element_size()), out.numel() if add else 0, None,
+                  self.lib.llmrs_embed_rows_add if add else self.lib.llmrs_embed_rows, self._stream(), _code(table.dtype), _p(out), _p(table), _p(tokens),
                   tokens.shape[0], table.shape[1], table.shape[0], float(scale))
 
     # out.flat[i] = mean + std * normal(seed, first + i): the same bits as the host library makes
@@ -334,6 +341,67 @@ class HipKernels(Kernels):
         self._run(f"rmsnorm {n}x{x.shape[1]}", n * x.shape[1] * (4 + out.element_size()) + x.shape[1] * 4, 5 * n * x.shape[1], None,
                   self.lib.llmrs_rmsnorm, self._stream(), _code(out.dtype), _p(out), _p(x), _p(weight), _p(rows),
                   n, x.shape[1], eps)
+
+    def dyt(self, out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, alpha: torch.Tensor,
+            rows: Optional[torch.Tensor] = None, second=None) -> None:
+        """out[i, :] = tanh(alpha * x[rows[i] or i, :]) * weight + bias; alpha is one number on the device.
+        second = (out2, weight2, bias2, alpha2): a second such norm of the same rows (every row), in the same pass."""
+        n, D = out.shape
+        assert x.dtype == weight.dtype == bias.dtype == alpha.dtype == torch.float32 and x.is_contiguous() and out.is_contiguous()
+        assert x.shape[1] == D == weight.numel() == bias.numel() and alpha.numel() == 1
+        assert (rows is None and n == x.shape[0]) or (rows is not None and rows.dtype == torch.int32 and rows.shape[0] == n)
+        out2 = w2 = b2 = a2 = None
+        if second is not None:
+            out2, w2, b2, a2 = second
+            assert rows is None and out2.shape == out.shape and out2.dtype == out.dtype and out2.is_contiguous()
+            assert w2.dtype == b2.dtype == a2.dtype == torch.float32 and w2.numel() == b2.numel() == D and a2.numel() == 1
+        outs = 1 if second is None else 2
+        self._run(f"dyt {n}x{D}" + (" twice" if second is not None else ""), n * D * (4 + outs * out.element_size()), 12 * outs * n * D, None,
+                  self.lib.llmrs_dyt, self._stream(), _code(out.dtype), _p(out), _p(x), _p(weight), _p(bias), _p(alpha), _p(rows),
+                  n, D, _p(out2), _p(w2), _p(b2), _p(a2))
+
+    def conv_state_update(self, sums: torch.Tensor, state: torch.Tensor, q_starts, slots, channels: int, taps: int) -> None:
+        """state [slots, >= (taps - 1) * channels] float32 becomes each request's last taps - 1 rows of (old state, this
+        step's rows of sums [T, channels]): what a causal convolution over `taps` taps reads before an entry's first token."""
+        assert sums.dtype == state.dtype == torch.float32 and sums.stride(1) == 1 and sums.shape[1] == channels
+        assert state.stride(-1) == 1 and state.shape[1] >= (taps - 1) * channels and q_starts.dtype == slots.dtype == torch.int32
+        self._run("conv_state", 2 * slots.numel() * (taps - 1) * channels * 4, 0, None, self.lib.llmrs_conv_state_update,
+                  self._stream(), _p(sums), sums.stride(0), _p(state), state.stride(0), _p(q_starts), _p(slots), slots.numel(), channels, taps)
+
+    def sigmoid_gate(self, o: torch.Tensor, gate: torch.Tensor, per: int) -> None:
+        """o[t, j] *= sigmoid(gate[t, j // per]) in place; gate float32 (a product's sums), the sigmoid and the product 32-bit."""
+        T, N = o.shape
+        assert gate.dtype == torch.float32 and o.stride(1) == 1 and gate.stride(1) == 1 and gate.shape[0] == T
+        assert per >= 1 and N % per == 0 and gate.shape[1] == N // per
+        self._run(f"sigmoid_gate {T}x{N}", T * N * 2 * o.element_size() + T * (N // per) * 4, 6 * T * N, None, self.lib.llmrs_sigmoid_gate,
+                  self._stream(), _code(o.dtype), _p(o), o.stride(0), _p(gate), gate.stride(0), T, N, per)
+
+    def latent_finish(self, sums: torch.Tensor, q: torch.Tensor, q_size: int, rank: int, weight: torch.Tensor, eps: float, slot_map,
+                      k_cache: torch.Tensor, v_cache: torch.Tensor, page_size: int, num_pages: int, write: bool) -> None:
+        """sums [T, q | c | ...] float32 -> q [T, q_size] in the activation type, and c = rmsnorm(sums_c) * weight into the
+        cache's pages twice, as a row of `k_cache` [page][slot][rank] and as a column of `v_cache` [page][rank][slot]."""
+        T = sums.shape[0]
+        assert sums.dtype == weight.dtype == torch.float32 and sums.stride(1) == 1 and sums.shape[1] >= q_size + rank
+        assert q.shape == (T, q_size) and q.stride(1) == 1 and weight.numel() == rank
+        if write:
+            assert k_cache.dtype == v_cache.dtype == q.dtype and k_cache.is_contiguous() and v_cache.is_contiguous()
+            assert k_cache.numel() == v_cache.numel() == num_pages * page_size * rank and slot_map.dtype == torch.int32 and slot_map.shape[0] == T
+        self._run("latent_finish", T * (q_size + rank) * (4 + q.element_size()) + T * rank * q.element_size(), 4 * T * rank, None,
+                  self.lib.llmrs_latent_finish, self._stream(), _code(q.dtype), _p(sums), sums.stride(0), _p(q), q.stride(0), T, q_size,
+                  rank, _p(weight), float(eps), _p(slot_map), _p(k_cache), _p(v_cache), page_size, num_pages, int(write))
+
+    def head_product(self, a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gate: Optional[torch.Tensor] = None) -> None:
+        """Every head by its own matrix: out[t, h, :] = w[h] @ a[t, h, :] with w [heads, n_out, n_in] (each [out, in]),
+        a [T, heads * n_in], out [T, heads * n_out], both in w's type, sums in 32-bit; gate [T, heads] float32: the sums
+        of head h are multiplied by sigmoid(gate[t, h]) before the one rounding."""
+        H, n_out, n_in = w.shape
+        T = a.shape[0]
+        assert a.dtype == w.dtype == out.dtype and w.is_contiguous() and a.stride(1) == 1 and out.stride(1) == 1
+        assert a.shape[1] == H * n_in and out.shape == (T, H * n_out)
+        assert gate is None or (gate.dtype == torch.float32 and gate.shape == (T, H) and gate.stride(1) == 1)
+        self._run(f"head_product {T}x{H}x{n_out}x{n_in}", (T * H * (n_in + n_out) + H * n_in * n_out) * a.element_size(),
+                  2 * T * H * n_in * n_out, a.dtype, self.lib.llmrs_head_product, self._stream(), _code(a.dtype), _p(a), a.stride(0),
+                  _p(w), _p(out), out.stride(0), T, H, n_in, n_out, int(self.allow_mfma), _p(gate), 0 if gate is None else gate.stride(0))
 
     # out (epilogue) a @ w.T ; a: [M, K] rows may be strided, w: [N, K] dense
     def gemm(self, a, w: torch.Tensor, out: torch.Tensor, epilogue: int = EPI_STORE,
@@ -418,8 +486,9 @@ class HipKernels(Kernels):
 
     def attention(self, q, out, k_cache, v_cache, block_table, token_entry, positions, q_starts, seq_lens,
                   n_heads, n_kv_heads, head_dim, page_size, num_pages, window, scale, scratch=None, max_seq_len=0, n_single=-1,
-                  single_keys=0, value_dim=0, distance=None, softcap=0.0, keep_first=0) -> None:
-        """single_keys: how many keys the single-token entries see together (windows counted), 0 if unknown.
+                  single_keys=0, value_dim=0, distance=None, softcap=0.0, keep_first=0, sink=None) -> None:
+        """sink: float32 [n_heads] or None: the softmax's denominator of head h also holds exp(sink[h]), once for every
+        query (a key without a value; not scaled).  single_keys: how many keys the single-token entries see together (windows counted), 0 if unknown.
         value_dim: the width of a value where it is not a key's (0: the same).  distance: (r1, r2), float32 [n_heads]
         each: r1[h] * ln(1 + r2[h] * (i - j)) is taken off the scaled score of query i and key j.  softcap > 0: the
         scaled score s becomes softcap * tanh(s / softcap).  keep_first: with a window, the request's first so many
@@ -428,10 +497,10 @@ class HipKernels(Kernels):
         assert block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous()
         v_dim = int(value_dim) or head_dim
         assert k_cache.numel() == num_pages * n_kv_heads * page_size * head_dim and v_cache.numel() == num_pages * n_kv_heads * page_size * v_dim
-        if v_dim != head_dim or distance is not None or softcap > 0 or (keep_first > 0 and window > 0):
+        if v_dim != head_dim or distance is not None or softcap > 0 or (keep_first > 0 and window > 0) or sink is not None:
             return self._attention_ext(q, out, k_cache, v_cache, block_table, token_entry, positions, q_starts, seq_lens, n_heads,
                                        n_kv_heads, head_dim, page_size, num_pages, window, scale, scratch, max_seq_len, n_single,
-                                       single_keys, v_dim, distance, softcap, keep_first)
+                                       single_keys, v_dim, distance, softcap, keep_first, sink)
         T = q.shape[0]
         assert token_entry.shape[0] == T and positions.shape[0] == T and out.shape[0] == T
         moved = flops = 0
@@ -450,8 +519,9 @@ class HipKernels(Kernels):
 
     def _attention_ext(self, q, out, k_cache, v_cache, block_table, token_entry, positions, q_starts, seq_lens, n_heads,
                        n_kv_heads, head_dim, page_size, num_pages, window, scale, scratch, max_seq_len, n_single, single_keys,
-                       v_dim, distance, softcap=0.0, keep_first=0) -> None:
+                       v_dim, distance, softcap=0.0, keep_first=0, sink=None) -> None:
         T = q.shape[0]
+        assert sink is None or (sink.dtype == torch.float32 and sink.numel() == n_heads and sink.is_contiguous())
         assert token_entry.shape[0] == T and positions.shape[0] == T and out.shape[0] == T
         r1 = r2 = None
         if distance is not None:
@@ -469,7 +539,7 @@ class HipKernels(Kernels):
                   _p(block_table), block_table.shape[1], _p(token_entry), _p(positions), _p(q_starts), _p(seq_lens),
                   block_table.shape[0], T, n_heads, n_kv_heads, head_dim, page_size, num_pages, window, scale,
                   _p(scratch), 0 if scratch is None else scratch.numel() * scratch.element_size(), int(max_seq_len),
-                  int(n_single), int(single_keys), int(self.allow_mfma), v_dim, _p(r1), _p(r2), float(softcap), int(keep_first))
+                  int(n_single), int(single_keys), int(self.allow_mfma), v_dim, _p(r1), _p(r2), float(softcap), int(keep_first), _p(sink))
 
     # out[i, :] = weight * groupnorm(sum_s w_in[s] * x[s][rows[i] or i, :]); x: [T, D] or [S, T, D] float32
     def group_rmsnorm(self, out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, eps: float, groups: int,
@@ -515,10 +585,26 @@ class HipKernels(Kernels):
 
     def qkv_finish(self, sums: torch.Tensor, bias: Optional[torch.Tensor], q: torch.Tensor, slot_map, k_cache, v_cache,
                    n_heads: int, n_kv_heads: int, head_dim: int, v_dim: int, page_size: int, num_pages: int, write_kv: bool,
-                   eps: float, positions: Optional[torch.Tensor] = None, inv_freq: Optional[torch.Tensor] = None, rotary_dim: int = 0) -> None:
+                   eps: float, positions: Optional[torch.Tensor] = None, inv_freq: Optional[torch.Tensor] = None, rotary_dim: int = 0,
+                   q_weight: Optional[torch.Tensor] = None, k_weight: Optional[torch.Tensor] = None, gain: float = 1.0, conv=None) -> None:
         """sums [T, q | k | v] float32 -> q [T, heads * head_dim] (activation type) and the cache's pages: biases
-        added, q and k divided by their root mean square over the head (eps > 0), then (rotary_dim > 0) their features
-        (2i, 2i + 1) turned by positions[t] * inv_freq[i]; one rounding on the way out."""
+        added, q and k divided by their root mean square over the head (eps > 0) and multiplied by q_weight / k_weight
+        [head_dim] (if given), then (rotary_dim > 0) their features (2i, 2i + 1) turned by positions[t] * inv_freq[i],
+        cosine and sine times `gain`; one rounding on the way out.
+        conv = (taps [columns, K] float32, state [slots, >= (K - 1) * columns] float32 or None when K == 1, q_starts, slots,
+        token_entry): every column first passes a causal convolution over its K taps, the last tap the token's own; rows
+        before an entry's first token come from the request's state (which `conv_state_update` brings up to date afterwards)."""
+        taps = state = q_starts = slots = token_entry = None
+        n_taps = n_entries = 0
+        if conv is not None:
+            taps, state, q_starts, slots, token_entry = conv
+            n_taps, n_entries = taps.shape[1], slots.numel()
+            assert taps.dtype == torch.float32 and taps.is_contiguous() and taps.shape[0] == sums.shape[1]
+            assert q_starts.dtype == slots.dtype == token_entry.dtype == torch.int32 and token_entry.numel() == sums.shape[0]
+            assert n_taps == 1 or (state is not None and state.dtype == torch.float32 and state.stride(-1) == 1
+                                   and state.shape[1] >= (n_taps - 1) * sums.shape[1])
+        for w in (q_weight, k_weight):
+            assert w is None or (w.dtype == torch.float32 and w.numel() == head_dim and w.is_contiguous() and eps > 0)
         if rotary_dim:
             assert positions.dtype == torch.int32 and positions.shape[0] == sums.shape[0] and inv_freq.dtype == torch.float32
             assert inv_freq.shape[0] == rotary_dim // 2 and inv_freq.is_contiguous() and rotary_dim % 2 == 0 and rotary_dim <= head_dim
@@ -533,7 +619,9 @@ class HipKernels(Kernels):
         self._run("qkv_finish", T * width * (4 + q.element_size()), 4 * T * width, None, self.lib.llmrs_qkv_finish,
                   self._stream(), _code(q.dtype), _p(sums), sums.stride(0), _p(bias), _p(q), q.stride(0), _p(slot_map),
                   _p(k_cache), _p(v_cache), T, n_heads, n_kv_heads, head_dim, v_dim, page_size, num_pages, int(write_kv), float(eps),
-                  _p(positions) if rotary_dim else None, _p(inv_freq) if rotary_dim else None, int(rotary_dim))
+                  _p(positions) if rotary_dim else None, _p(inv_freq) if rotary_dim else None, int(rotary_dim),
+                  _p(q_weight), _p(k_weight), float(gain), _p(taps), int(n_taps), _p(state) if n_taps > 1 else None,
+                  state.stride(0) if n_taps > 1 else 0, _p(q_starts), _p(slots), _p(token_entry), int(n_entries))
 
     def add_bias_rows(self, rows: torch.Tensor, bias: torch.Tensor) -> None:
         """rows[t, :] += bias; both float32."""

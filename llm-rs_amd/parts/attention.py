@@ -16,9 +16,15 @@ keys), `bias` (q, k and v have biases), `qk_norm_eps` (q and k are divided by th
 with this eps, no weight), `distance` = "log" (a per-head penalty r1 ln(1 + r2 (i - j)) taken off the scaled score,
 with the head's numbers in two tensors), `softcap` (the scaled score s becomes softcap tanh(s / softcap)),
 `keep_first` (with a window, the request's first so many keys stay visible at their true positions; their pages stay in
-the cache), `o_bias` (the output projection has a bias), `names` (the leaves of the tensors' names).  With any of them
-the q/k/v product leaves 32-bit sums, and one kernel adds the biases, norms q and k, rotates them (a rotation that the
-kernels fuse, angles in 32-bit) and writes k and v into their pages.
+the cache), `o_bias` (the output projection has a bias), `conv` (q, k and v each pass a causal convolution over that many
+taps per channel right after the projection, the last tap the current token's, no bias, no activation; the request's
+last conv - 1 projected rows are kept in its slot beside the pages), `qk_norm_weight` (the q/k norm multiplies by a
+weight of head_dim numbers, one tensor for q and one for k, shared by the heads), a rotation with a `gain` (cosine and
+sine both enlarged: the position encoding says so), `gate` = "feature" | "head" (the heads' outputs are multiplied by
+sigmoid(Wg x), one gate for every feature of every head or one for each head, before the output projection; the gate's
+rows ride in the q/k/v product), `names` (the leaves of the tensors' names).  With any of them the q/k/v product leaves
+32-bit sums, and one kernel convolves, adds the biases, norms q and k, rotates them (a rotation that the kernels fuse,
+angles in 32-bit) and writes k and v into their pages.
 
 The rotation kernels pair neighbours (2i, 2i+1).  Where the encoding pairs
 (i, i + rotary_dim/2), the rows of Wq and Wk are reordered within each head at
@@ -32,12 +38,48 @@ import math
 
 import torch
 
-from ..cache.spec import PagedKV
+from ..cache.spec import FixedState, PagedKV
 from ..kernels import EPI_ACCUM_F32, EPI_STORE, EPI_STORE_F32, kernels
 from .base import Mixer, TensorSpec, build_position, place, register_mixer
 
 
-class Attention(Mixer):
+class KeyedBySplitChunk:
+    """For mixers that call `kernels().attention`: what their recordings are keyed by.  The mixer sets
+    `recording_signature = ("attention", kv_heads, head_dim, window)`, the shape of the cache its queries walk."""
+
+    # The kernel library shares the decoding requests' keys out over waves in chunks whose length it chooses by
+    # how many keys the step sees (`single_keys`).  A recorded step holds the chunk it was recorded with, so the
+    # chunk is part of what recordings are keyed by; and since recording a step again costs about as much as a step
+    # while a chunk that is no longer the best one costs a few per cent of the attention, a batch keeps the figure
+    # it was recorded with until the rule has asked for another chunk this many steps in a row.
+    chunk_patience = 256
+
+    def recording_key(self, ctx):
+        k = kernels()
+        if not ctx.n_single:
+            return 0
+        keys = ctx.single_keys(self.recording_signature[3])
+        want = k.attention_split_chunk(ctx.n_single, self.recording_signature[1], self.recording_signature[2], ctx.max_seq_len, keys)
+        held = ctx.part_state.setdefault(self.recording_signature, {})
+        at = (ctx.n_single, ctx.max_seq_len)
+        now = held.get(at)             # [chunk, a number of keys that gives it, steps in a row that wanted another, step]
+        if now is None or want == now[0] or now[2] >= self.chunk_patience:
+            now = held[at] = [want, keys, 0, ctx.serial]
+        else:
+            now[2] += 1
+            now[3] = ctx.serial
+        return now[0]
+
+    def _keys_for_the_split(self, ctx) -> int:
+        if not ctx.n_single:
+            return 0
+        now = ctx.part_state.get(self.recording_signature, {}).get((ctx.n_single, ctx.max_seq_len))
+        if now is not None and now[3] == ctx.serial:      # this step was keyed by a chunk: the figure that gives it
+            return now[1]
+        return ctx.single_keys(self.recording_signature[3])
+
+
+class Attention(KeyedBySplitChunk, Mixer):
     graph_safe = True
 
     def __init__(self, spec, dtype):
@@ -72,19 +114,32 @@ class Attention(Mixer):
         self.has_o_bias = bool(p.get("o_bias", False))
         if self.softcap < 0 or self.keep_first < 0:
             raise ValueError("softcap and keep_first must not be negative")
+        self.taps = int(p.get("conv") or 0)
+        self.qk_norm_weight = bool(p.get("qk_norm_weight", False))
+        self.gate = p.get("gate")
+        if self.gate not in (None, "feature", "head"):
+            raise ValueError(f"unknown output gate {self.gate!r} (known: feature, head)")
+        if self.qk_norm_weight and not self.qk_norm_eps > 0:
+            raise ValueError("a q/k norm with a weight needs its eps (qk_norm_eps)")
+        if self.taps > 0 and (not self.kv_proj or self.has_bias):
+            raise ValueError("convolutions on q, k and v go with neither biases nor a cache that another mixer wrote")
+        self.gate_size = {None: 0, "feature": self.o_size, "head": self.heads}[self.gate]
+        self.gain = float(getattr(self.position, "gain", 1.0)) if self.position is not None else 1.0
         # q and k are prepared by a kernel of their own between the product and attention
         self.prepared = (self.has_bias or self.qk_norm_eps > 0 or self.distance is not None or self.value_dim != self.head_dim
-                         or self.softcap > 0 or self.keep_first > 0)
+                         or self.softcap > 0 or self.keep_first > 0 or self.taps > 1 or self.gate is not None or self.gain != 1.0)
         if self.prepared and self.position is not None and self.position.rotary() is None:
             raise ValueError("a position encoding that is no rotation together with biases, a q/k norm, a distance penalty, a soft cap, "
                              "kept first keys or values of another width is not built")
         leaves = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
                   "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias", "o_bias": "o_proj.bias", "r1": "r1", "r2": "r2",
-                  **(p.get("names") or {})}
+                  "q_norm": "q_norm.weight", "k_norm": "k_norm.weight", "q_conv": "q_conv.weight", "k_conv": "k_conv.weight",
+                  "v_conv": "v_conv.weight", "gate": "gate_proj.weight", **(p.get("names") or {})}
         self.names = {key: self.name(leaf) for key, leaf in leaves.items()}
         self.w_qkv = None
         self.w_o = None
         self.bias = self.o_bias = self.r1 = self.r2 = None
+        self.q_norm = self.k_norm = self.conv = None
         # Set by a part that holds this mixer and adds the output projection's bias itself, in a pass over the output
         # that it makes anyway (it reads the bias from `o_bias`): `forward` then leaves the bias out.
         self.output_bias_left_to_holder = False
@@ -105,6 +160,16 @@ class Attention(Mixer):
         if self.distance is not None:
             t[n["r1"]] = TensorSpec((self.heads,), "normal:0.5:0.2")
             t[n["r2"]] = TensorSpec((self.heads,), "normal:0.5:0.05")     # 1 + r2 (i - j) must stay positive
+        if self.qk_norm_weight:
+            t[n["q_norm"]] = TensorSpec((self.head_dim,), "norm")
+            if self.kv_proj:
+                t[n["k_norm"]] = TensorSpec((self.head_dim,), "norm")
+        if self.taps > 0:
+            t[n["q_conv"]] = TensorSpec((self.q_size, self.taps), "normal:0.0:0.4")
+            t[n["k_conv"]] = TensorSpec((self.kv_size, self.taps), "normal:0.0:0.4")
+            t[n["v_conv"]] = TensorSpec((self.v_size, self.taps), "normal:0.0:0.4")
+        if self.gate is not None:
+            t[n["gate"]] = TensorSpec((self.gate_size, self.hidden))
         return t
 
     def _pair_neighbours(self, w: torch.Tensor, heads: int, undo: bool = False) -> torch.Tensor:
@@ -125,8 +190,17 @@ class Attention(Mixer):
         parts = [self._pair_neighbours(get("q"), self.heads)]
         if self.kv_proj:
             parts += [self._pair_neighbours(get("k"), self.kv_heads), get("v")]
+        self.qkv_width = sum(w.shape[0] for w in parts)
+        if self.gate is not None:       # the gate's rows behind q | k | v: one product for all that reads the mixer's input
+            parts.append(get("gate"))
         self.w_qkv = torch.cat(parts, dim=0).contiguous()
         self.w_o = get("o")
+        if self.qk_norm_weight:         # (a head's features are listed in the order its rotation pairs them in)
+            self.q_norm = self._pair_neighbours(get32("q_norm").unsqueeze(1), 1).squeeze(1).contiguous()
+            self.k_norm = self._pair_neighbours(get32("k_norm").unsqueeze(1), 1).squeeze(1).contiguous() if self.kv_proj else None
+        if self.taps > 0:               # the taps of q | k | v one under the other, as the product's columns are
+            self.conv = torch.cat([self._pair_neighbours(get32("q_conv"), self.heads), self._pair_neighbours(get32("k_conv"), self.kv_heads),
+                                   get32("v_conv")], dim=0).contiguous()
         if self.has_bias:       # added to the 32-bit sums: kept in 32-bit, side by side as the product's columns are (and reordered as its rows are)
             pair = lambda b, heads: self._pair_neighbours(b.unsqueeze(1), heads).squeeze(1)
             self.bias = torch.cat([pair(get32("q_bias"), self.heads)] +
@@ -142,8 +216,19 @@ class Attention(Mixer):
         w = self.w_qkv.cpu()
         n = self.names
         out = {n["q"]: self._pair_neighbours(w[:self.q_size], self.heads, undo=True).contiguous(), n["o"]: self.w_o.cpu()}
+        if self.gate is not None:
+            out[n["gate"]] = w[self.qkv_width:].contiguous()
+        if self.qk_norm_weight:
+            out[n["q_norm"]] = self._pair_neighbours(self.q_norm.cpu().unsqueeze(1), 1, undo=True).squeeze(1).contiguous()
+            if self.kv_proj:
+                out[n["k_norm"]] = self._pair_neighbours(self.k_norm.cpu().unsqueeze(1), 1, undo=True).squeeze(1).contiguous()
+        if self.taps > 0:
+            c = self.conv.cpu()
+            out[n["q_conv"]] = self._pair_neighbours(c[:self.q_size], self.heads, undo=True).contiguous()
+            out[n["k_conv"]] = self._pair_neighbours(c[self.q_size:self.q_size + self.kv_size], self.kv_heads, undo=True).contiguous()
+            out[n["v_conv"]] = c[self.q_size + self.kv_size:].contiguous()
         if self.kv_proj:
-            k, v = w[self.q_size:self.q_size + self.kv_size], w[self.q_size + self.kv_size:]
+            k, v = w[self.q_size:self.q_size + self.kv_size], w[self.q_size + self.kv_size:self.qkv_width]
             out[n["k"]] = self._pair_neighbours(k, self.kv_heads, undo=True).contiguous()
             out[n["v"]] = v.contiguous()
         if self.has_bias:
@@ -160,23 +245,39 @@ class Attention(Mixer):
         return out
 
     def cache_need(self):
-        return PagedKV(self.kv_heads, self.head_dim, self.window, self.value_dim if self.value_dim != self.head_dim else 0, self.keep_first)
+        pages = PagedKV(self.kv_heads, self.head_dim, self.window, self.value_dim if self.value_dim != self.head_dim else 0, self.keep_first)
+        if self.taps > 1:       # beside the pages, in the request's slot: the last conv - 1 rows of q | k | v as projected, 32-bit
+            return (pages, FixedState(((self.taps - 1) * self.qkv_columns,), torch.float32))
+        return pages
+
+    @property
+    def qkv_columns(self) -> int:
+        return self.q_size + (self.kv_size + self.v_size if self.kv_proj else 0)
 
     def _forward_prepared(self, ctx, x, h, cache):
-        """The product's 32-bit sums -> biases, unit norm and rotation of q and k, cache write -> attention with the
-        distance penalty, the soft cap and the kept first keys."""
+        """The product's 32-bit sums -> convolution, biases, norm and rotation of q and k, cache write -> attention with
+        the distance penalty, the soft cap and the kept first keys -> the output gate -> the output projection."""
         k = kernels()
         T = x.shape[0]
+        conv_state = None
+        if cache.kind == "several":          # pages, and the convolutions' last inputs in the request's slot
+            cache, conv_state = cache.parts[0], cache.parts[1].state
         write = self.kv_proj and cache.writes
         n_kv = self.kv_heads if self.kv_proj else 0
         g = cache.group
+        C = self.qkv_columns
         sums = ctx.workspace("attn.sums", (T, self.w_qkv.shape[0]), torch.float32)
         k.gemm(x, self.w_qkv, sums, EPI_STORE_F32, ctx.gemm_workspace(x, self.w_qkv))
         q = ctx.workspace("attn.qkv", (T, self.q_size), self.dtype)
         rotary = self.position.rotary() if self.position is not None else None
         inv_freq, rotary_dim = (None, 0) if rotary is None else rotary[:2]
-        k.qkv_finish(sums, self.bias, q, ctx.slot_maps[g], cache.k, cache.v, self.heads, n_kv, self.head_dim, self.value_dim,
-                     cache.page_size, cache.num_pages, write, self.qk_norm_eps, ctx.positions, inv_freq, rotary_dim)
+        # (one tap: every channel times its number, and nothing to remember)
+        conv = (self.conv, conv_state, ctx.q_starts, ctx.slots, ctx.token_entry) if self.taps > 0 else None
+        k.qkv_finish(sums[:, :C], self.bias, q, ctx.slot_maps[g], cache.k, cache.v, self.heads, n_kv, self.head_dim, self.value_dim,
+                     cache.page_size, cache.num_pages, write, self.qk_norm_eps, ctx.positions, inv_freq, rotary_dim,
+                     q_weight=self.q_norm, k_weight=self.k_norm, gain=self.gain, conv=conv)
+        if self.taps > 1:
+            k.conv_state_update(sums[:, :C], conv_state, ctx.q_starts, ctx.slots, C, self.taps)
         o = ctx.workspace("attn.out", (T, self.o_size), self.dtype)
         need = k.attention_scratch_floats(ctx.n_entries, self.heads, max(self.head_dim, self.value_dim), ctx.max_seq_len,
                                           self.kv_heads, ctx.n_single) if ctx.n_single else 0
@@ -185,6 +286,8 @@ class Attention(Mixer):
                     self.heads, self.kv_heads, self.head_dim, cache.page_size, cache.num_pages, self.window, self.scale,
                     scratch, ctx.max_seq_len, ctx.n_single, self._keys_for_the_split(ctx), value_dim=self.value_dim,
                     distance=None if self.distance is None else (self.r1, self.r2), softcap=self.softcap, keep_first=self.keep_first)
+        if self.gate is not None:
+            k.sigmoid_gate(o, sums[:, self.qkv_width:], 1 if self.gate == "feature" else self.value_dim)
         k.gemm(o, self.w_o, h, EPI_ACCUM_F32, ctx.gemm_workspace(o, self.w_o))
         if self.has_o_bias and not self.output_bias_left_to_holder:
             k.add_bias_rows(h, self.o_bias)
@@ -196,37 +299,6 @@ class Attention(Mixer):
         # the q/k/v product norms its rows itself where it is the fused kernel: a rotation it applies (or none)
         fused = self.position is None or self.position.rotary() is not None
         return fused and kernels().product_norms_its_rows(rows, self.w_qkv.shape[0], self.hidden, self.dtype)
-
-    # The kernel library shares the decoding requests' keys out over waves in chunks whose length it chooses by
-    # how many keys the step sees (`single_keys`).  A recorded step holds the chunk it was recorded with, so the
-    # chunk is part of what recordings are keyed by; and since recording a step again costs about as much as a step
-    # while a chunk that is no longer the best one costs a few per cent of the attention, a batch keeps the figure
-    # it was recorded with until the rule has asked for another chunk this many steps in a row.
-    chunk_patience = 256
-
-    def recording_key(self, ctx):
-        k = kernels()
-        if not ctx.n_single:
-            return 0
-        keys = ctx.single_keys(self.window)
-        want = k.attention_split_chunk(ctx.n_single, self.kv_heads, self.head_dim, ctx.max_seq_len, keys)
-        held = ctx.part_state.setdefault(self.recording_signature, {})
-        at = (ctx.n_single, ctx.max_seq_len)
-        now = held.get(at)             # [chunk, a number of keys that gives it, steps in a row that wanted another, step]
-        if now is None or want == now[0] or now[2] >= self.chunk_patience:
-            now = held[at] = [want, keys, 0, ctx.serial]
-        else:
-            now[2] += 1
-            now[3] = ctx.serial
-        return now[0]
-
-    def _keys_for_the_split(self, ctx) -> int:
-        if not ctx.n_single:
-            return 0
-        now = ctx.part_state.get(self.recording_signature, {}).get((ctx.n_single, ctx.max_seq_len))
-        if now is not None and now[3] == ctx.serial:      # this step was keyed by a chunk: the figure that gives it
-            return now[1]
-        return ctx.single_keys(self.window)
 
     def forward(self, ctx, x, h, cache):
         if self.prepared:

@@ -2,7 +2,8 @@
 (src/arch/llama.rs:152-170).  Another arrangement (one norm for two parallel
 halves, norms after the parts) is another subclass of `Block`, registered under
 its own name; the parts it needs beyond these four come under the names the
-layer's spec gives them in `extra`.  "sandwich": a norm before and after each half."""
+layer's spec gives them in `extra`.  "sandwich": a norm before and after each half.
+"parallel": both halves read the stream as it was, each through a norm of its own."""
 from __future__ import annotations
 
 import torch
@@ -68,3 +69,38 @@ class SandwichBlock(Block):
 
 
 register_block("sandwich", SandwichBlock)
+
+
+class ParallelBlock(Block):
+    """Both halves read the same stream, each through its own norm, and both add into it:
+    h <- h + mixer(mixer_norm(h)) + feed_forward(feed_forward_norm(h)).  The two norms run before either half touches
+    the stream (in one launch where the norms can: `forward_with`); the sums are 32-bit.  A layer may have no
+    feed-forward."""
+    needs = ("mixer", "mixer_norm")
+
+    def __init__(self, named):
+        super().__init__(named)
+        if self.feed_forward is not None and self.feed_forward_norm is None:
+            raise ValueError("block arrangement ParallelBlock needs the parts feed_forward_norm")
+
+    def forward(self, ctx, h, cache):
+        T, D = h.shape
+        ctx.note_left(h, None)
+        ctx.upcoming_norm = None
+        x = ctx.workspace("block.x", (T, D), self.mixer.dtype)
+        if self.feed_forward is None:
+            self.mixer_norm.forward(ctx, h, x)
+            self.mixer.forward(ctx, x, h, cache)
+        else:
+            x2 = ctx.workspace("block.x2", (T, D), self.feed_forward.dtype)
+            together = getattr(self.mixer_norm, "forward_with", None)
+            if together is None or not together(ctx, h, x, self.feed_forward_norm, x2):
+                self.mixer_norm.forward(ctx, h, x)
+                self.feed_forward_norm.forward(ctx, h, x2)
+            self.mixer.forward(ctx, x, h, cache)
+            self.feed_forward.forward(ctx, x2, h)
+        ctx.note_left(h, None)
+        ctx.upcoming_norm = None
+
+
+register_block("parallel", ParallelBlock)

@@ -1,4 +1,4 @@
-"""RMSNorm(size, eps): y = x / sqrt(mean(x^2) + eps) * weight, computed in 32-bit,
+"""Norms.  RMSNorm(size, eps): y = x / sqrt(mean(x^2) + eps) * weight, computed in 32-bit,
 the weight multiplying directly.  Reference: rms_norm_batch
 (shaders/ops.metal:970-1003), used at src/arch/llama.rs:152,164,135."""
 from __future__ import annotations
@@ -101,3 +101,47 @@ class GroupRMSNorm(Norm):
 
 
 register_norm("group_rmsnorm", GroupRMSNorm)
+
+
+class DynamicTanh(Norm):
+    """Dynamic tanh(size): y = tanh(alpha x) weight + bias, with one scalar alpha for the whole row, a weight and a bias
+    per feature; nothing is summed over the row (no mean, no variance, no eps).  32-bit throughout, one rounding on the
+    way out.  Tensors: the weight under the prefix itself, the bias under `<prefix>.b`, the scalar under
+    `<prefix>.alpha` (`names` gives other leaves).  Two such norms of the same rows run in one launch that reads the
+    rows once (`forward_with`)."""
+    graph_safe = True
+
+    def __init__(self, spec, dtype):
+        super().__init__(spec, dtype)
+        self.size = int(spec.params["size"])
+        leaves = {"weight": "", "bias": "b", "alpha": "alpha", **(spec.params.get("names") or {})}
+        self.names = {key: (self.name(leaf) if leaf else self.prefix) for key, leaf in leaves.items()}
+        self.weight = self.bias = self.alpha = None
+
+    def tensors(self):
+        n = self.names
+        return {n["weight"]: TensorSpec((self.size,), "norm"), n["bias"]: TensorSpec((self.size,), "normal:0.0:0.1"),
+                n["alpha"]: TensorSpec((), "normal:0.6:0.1")}
+
+    def load(self, tensors, device):
+        get = lambda key: place(tensors[self.names[key]], device, torch.float32)
+        self.weight, self.bias = get("weight"), get("bias")
+        self.alpha = get("alpha").reshape(1)            # stays on the device: the kernel reads it there
+
+    def export(self):
+        n = self.names
+        return {n["weight"]: self.weight.cpu(), n["bias"]: self.bias.cpu(), n["alpha"]: self.alpha.cpu().reshape(())}
+
+    def forward(self, ctx, h, out, rows=None):
+        kernels().dyt(out, h, self.weight, self.bias, self.alpha, rows)
+
+    def forward_with(self, ctx, h, out, other, other_out) -> bool:
+        """out = this norm of every row of h and other_out = `other`'s, in one launch; False when `other` is of
+        another kind (the caller then runs the two one after the other)."""
+        if not isinstance(other, DynamicTanh) or other.size != self.size:
+            return False
+        kernels().dyt(out, h, self.weight, self.bias, self.alpha, None, second=(other_out, other.weight, other.bias, other.alpha))
+        return True
+
+
+register_norm("dyt", DynamicTanh)

@@ -9,6 +9,11 @@ with wavelength = 2 pi / freq and L = original_max_position_embeddings,
   wavelength < L / high_freq_factor : freq kept
   wavelength > L / low_freq_factor  : freq / factor
   between: s = (L / wavelength - low) / (high - low), freq <- (1 - s) freq / factor + s freq.
+"ramp" scaling (factor, original, fast, slow) bends the frequencies by the index of the pair instead: with
+  d(t) = rotary_dim ln(original / (2 pi t)) / (2 ln theta),  lo = max(floor(d(fast)), 0),  hi = min(ceil(d(slow)), rotary_dim - 1),
+  r_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1):  freq_i <- freq_i / factor r_i + freq_i (1 - r_i),
+and enlarges the turned features: cosine and sine are both multiplied by `gain` = 0.1 ln(factor) + 1 (the features
+that are not turned pass as they are, so the gain is no part of the score's scale).
 The table is made once on the host in double precision and rounded to float32;
 the kernel multiplies float(position) by it in 32-bit.
 """
@@ -22,11 +27,30 @@ import torch
 from .base import PositionEncoding, register_position
 
 
+def _ramp_bounds(rotary_dim: int, theta: float, scaling: Mapping):
+    original = float(scaling["original"])
+    d = lambda t: rotary_dim * math.log(original / (2.0 * math.pi * t)) / (2.0 * math.log(theta))
+    return max(math.floor(d(float(scaling["fast"]))), 0), min(math.ceil(d(float(scaling["slow"]))), rotary_dim - 1)
+
+
+def rope_gain(scaling: Optional[Mapping]) -> float:
+    """What cosine and sine are multiplied by: 1 for every scaling but "ramp"."""
+    if scaling is None or scaling.get("rope_type", "llama3") != "ramp":
+        return 1.0
+    return 0.1 * math.log(float(scaling["factor"])) + 1.0
+
+
 def rope_inv_freq(rotary_dim: int, theta: float, scaling: Optional[Mapping]) -> torch.Tensor:
     out = []
+    ramp = scaling is not None and scaling.get("rope_type", "llama3") == "ramp"
+    if ramp and rotary_dim > 0:
+        lo, hi = _ramp_bounds(rotary_dim, theta, scaling)
     for i in range(rotary_dim // 2):
         freq = theta ** (-2.0 * i / rotary_dim)
-        if scaling is not None:
+        if ramp:
+            r = min(max((i - lo) / max(hi - lo, 0.001), 0.0), 1.0)
+            freq = freq / float(scaling["factor"]) * r + freq * (1.0 - r)
+        elif scaling is not None:
             if scaling.get("rope_type", "llama3") != "llama3":
                 raise ValueError(f"unsupported rope scaling {scaling.get('rope_type')!r}")
             factor, low, high = float(scaling["factor"]), float(scaling["low_freq_factor"]), float(scaling["high_freq_factor"])
@@ -53,6 +77,7 @@ class RotaryEncoding(PositionEncoding):
             raise ValueError(f"unknown rotary layout {layout!r}")
         self.interleaved = layout == "interleaved"
         self.inv_freq = rope_inv_freq(self.rotary_dim, float(params["theta"]), params.get("scaling"))
+        self.gain = rope_gain(params.get("scaling")) if self.rotary_dim > 0 else 1.0
 
     def to(self, device):
         self.inv_freq = self.inv_freq.to(device)

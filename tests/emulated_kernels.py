@@ -17,8 +17,46 @@ EPI_STORE, EPI_STORE_F32, EPI_ACCUM_F32, EPI_SWIGLU = 0, 1, 2, 3
 class EmulatedKernels(Kernels):
     """(What `Kernels` answers by itself stays: no workspace, no scratch, nothing split.)"""
 
-    def embed_rows(self, out, table, tokens, scale=1.0):
-        out.copy_(table[tokens.long()].float() * scale)
+    def embed_rows(self, out, table, tokens, scale=1.0, add=False):
+        rows = table[tokens.long()].float() * scale
+        out.add_(rows) if add else out.copy_(rows)
+
+    def dyt(self, out, x, weight, bias, alpha, rows=None, second=None):
+        src = x if rows is None else x[rows.long()]
+        out.copy_((torch.tanh(alpha * src) * weight + bias).to(out.dtype))
+        if second is not None:
+            out2, w2, b2, a2 = second
+            out2.copy_((torch.tanh(a2 * src) * w2 + b2).to(out2.dtype))
+
+    def conv_state_update(self, sums, state, q_starts, slots, channels, taps):
+        for e in range(slots.numel()):
+            t0, t1 = int(q_starts[e]), int(q_starts[e + 1])
+            st = state[int(slots[e])]
+            old = st[:(taps - 1) * channels].view(taps - 1, channels)
+            old.copy_(torch.cat([old, sums[t0:t1, :channels]])[-(taps - 1):].clone())
+
+    def sigmoid_gate(self, o, gate, per):
+        g = torch.sigmoid(gate).repeat_interleave(per, dim=1)
+        o.copy_((o.float() * g).to(o.dtype))
+
+    def latent_finish(self, sums, q, q_size, rank, weight, eps, slot_map, k_cache, v_cache, page_size, num_pages, write):
+        q.copy_(sums[:, :q_size].to(q.dtype))
+        if not write:
+            return
+        c = sums[:, q_size:q_size + rank]
+        c = c / torch.sqrt((c * c).mean(-1, keepdim=True) + eps) * weight
+        kc, vc = k_cache.view(num_pages, page_size, rank), v_cache.view(num_pages, rank, page_size)
+        page, off = (slot_map // page_size).long(), (slot_map % page_size).long()
+        for t in range(sums.shape[0]):
+            kc[page[t], off[t], :] = c[t].to(kc.dtype)
+            vc[page[t], :, off[t]] = c[t].to(vc.dtype)
+
+    def head_product(self, a, w, out, gate=None):
+        H, n_out, n_in = w.shape
+        acc = torch.einsum("thi,hoi->tho", a.float().view(a.shape[0], H, n_in), w.float())
+        if gate is not None:
+            acc = acc * torch.sigmoid(gate)[:, :, None]
+        out.copy_(acc.reshape(a.shape[0], H * n_out).to(out.dtype))
 
     def scale_softcap_rows(self, logits, scale, cap):
         logits.mul_(scale)
@@ -109,7 +147,7 @@ class EmulatedKernels(Kernels):
 
     def attention(self, q, out, k_cache, v_cache, block_table, token_entry, positions, q_starts, seq_lens,
                   n_heads, n_kv_heads, head_dim, page_size, num_pages, window, scale, scratch=None, max_seq_len=0, n_single=-1,
-                  single_keys=0, value_dim=0, distance=None, softcap=0.0, keep_first=0):
+                  single_keys=0, value_dim=0, distance=None, softcap=0.0, keep_first=0, sink=None):
         T = q.shape[0]
         v_dim = value_dim or head_dim
         kc = k_cache.view(num_pages, n_kv_heads, page_size, head_dim).float()
@@ -132,7 +170,10 @@ class EmulatedKernels(Kernels):
                     s = softcap * torch.tanh(s / softcap)
                 if distance is not None:
                     s = s - distance[0][h] * torch.log1p(distance[1][h] * (pos - js).float())
-                p = torch.softmax(s, dim=0)
+                if sink is not None:         # a key without a value: it only enlarges the denominator
+                    p = torch.softmax(torch.cat([s, sink[h:h + 1]]), dim=0)[:-1]
+                else:
+                    p = torch.softmax(s, dim=0)
                 out[t, h * v_dim:(h + 1) * v_dim] = (p @ vals[:, g, :]).to(out.dtype)
 
     def group_rmsnorm(self, out, x, weight, eps, groups, rows=None, w_in=None, zero=None, combined=None, mix=None):
@@ -145,16 +186,31 @@ class EmulatedKernels(Kernels):
             zero.zero_()
 
     def qkv_finish(self, sums, bias, q, slot_map, k_cache, v_cache, n_heads, n_kv_heads, head_dim, v_dim, page_size, num_pages,
-                   write_kv, eps, positions=None, inv_freq=None, rotary_dim=0):
+                   write_kv, eps, positions=None, inv_freq=None, rotary_dim=0, q_weight=None, k_weight=None, gain=1.0, conv=None):
         T = sums.shape[0]
-        x = sums + bias if bias is not None else sums.clone()
+        if conv is not None:
+            taps, state, q_starts, slots, token_entry = conv
+            K, C = taps.shape[1], sums.shape[1]
+            x = torch.zeros_like(sums)
+            for e in range(slots.numel()):
+                t0, t1 = int(q_starts[e]), int(q_starts[e + 1])
+                before = state[int(slots[e])][:(K - 1) * C].view(K - 1, C) if K > 1 else sums[:0]
+                rows = torch.cat([before, sums[t0:t1]])
+                for j in range(K):
+                    x[t0:t1] += taps[:, j] * rows[j:j + t1 - t0]
+        else:
+            x = sums + bias if bias is not None else sums.clone()
         nq, nk = n_heads * head_dim, n_kv_heads * head_dim
         qk = x[:, :nq + nk].reshape(T, n_heads + n_kv_heads, head_dim)
         if eps > 0:
             qk = qk / torch.sqrt((qk * qk).mean(-1, keepdim=True) + eps)
+            if q_weight is not None:
+                qk[:, :n_heads] = qk[:, :n_heads] * q_weight
+            if k_weight is not None:
+                qk[:, n_heads:] = qk[:, n_heads:] * k_weight
         if rotary_dim:
             angle = positions.float()[:, None] * inv_freq[None, :]
-            cos, sin = torch.cos(angle)[:, None, :], torch.sin(angle)[:, None, :]
+            cos, sin = torch.cos(angle)[:, None, :] * gain, torch.sin(angle)[:, None, :] * gain
             a, b = qk[..., 0:rotary_dim:2].clone(), qk[..., 1:rotary_dim:2].clone()
             qk[..., 0:rotary_dim:2], qk[..., 1:rotary_dim:2] = a * cos - b * sin, b * cos + a * sin
         q.copy_(qk[:, :n_heads].reshape(T, nq).to(q.dtype))
