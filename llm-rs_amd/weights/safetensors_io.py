@@ -92,4 +92,4 @@ def write_safetensors(path: str, tensors: Dict[str, torch.Tensor], metadata: Dic
         f.write(blob)
         for name in order:
             t = tensors[name].detach().cpu().contiguous()
-            f.write(t.view(torch.uint8).numpy().tobytes() if t.numel() else b"")
+            f.write(t.reshape(-1).view(torch.uint8).numpy().tobytes() if t.numel() else b"")      # (a tensor without dimensions is one element)

@@ -146,11 +146,11 @@ def plain_latent_attention(h: torch.Tensor, w: Dict[str, torch.Tensor], m: dict,
     H, dk, dv = int(m["heads"]), int(m["dim"]), int(m["vdim"])
     q = rnd(h @ w["q"].T).view(T, H, dk)
     c = rnd(plain_rmsnorm(h @ w["dkv"].T, w["dkv.norm"], eps))
-    k = (c @ w["uk"].T).view(T, H, dk)
-    v = (c @ w["uv"].T).view(T, H, dv)
+    k = rnd(c @ w["uk"].T).view(T, H, dk)
+    v = rnd(c @ w["uv"].T).view(T, H, dv)
     scores = torch.einsum("ihd,jhd->hij", q, k) * float(m["scale"]) + plain_causal_mask(T, h.dtype)[None]
     p = plain_softmax_rows(scores, w["sink"])
-    o = torch.einsum("hij,jhd->ihd", p, v)                         # [T, H, dv]
+    o = rnd(torch.einsum("hij,jhd->ihd", p, v))                    # [T, H, dv]
     o = o * plain_sigmoid(h @ w["g"].T)[:, :, None]                # one gate per head
     return rnd(o.reshape(T, H * dv)) @ w["o"].T
 
