@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Decode and prefill throughput of the engine on one MI355X.
 
-    python bench.py --gpus 1 --steps K --warmup W [--workload decode8b|serve1b|mixed70b|sizes|sizes1b|prompts|long|widths|portions|tuvodra|lilatar]
+    python bench.py --gpus 1 --steps K --warmup W [--workload decode8b|serve1b|mixed70b|sizes|sizes1b|prompts|long|widths|portions|tuvodra|lilatar|vivisun]
 
 The default run (`decode8b`) is the Llama-3.1-8B shape with random bfloat16 weights: 8
 requests, each with 2,048 tokens of context in the cache, decode K steps through the
@@ -37,6 +37,8 @@ The other workloads print one line of the same form each:
             2,048 tokens and a decode step of 8 requests over 2,048 tokens for each.
   lilatar   the same for the Lilatar decoder (linear attention, windowed attention beside a gated delta rule,
             dense and routed squared-relu feed-forwards).
+  vivisun   the same for the Vivisun decoder (dynamic-tanh norms, both halves of a layer on the same stream; attention
+            with convolved q/k/v, normed and half-rotated heads and a gate, in turns with latent attention with a sink).
 With LLM_PERF set in the environment every kernel call is timed by itself and a table
 by kernel goes to stderr (the reference's switch, src/backend/metal/mod.rs:235,321-400).
 """
@@ -67,7 +69,7 @@ LLAMA_8B = _llama(32, 4096, 32, 8, 128, 14336, 8.0, False)
 LLAMA_1B = _llama(16, 2048, 32, 8, 64, 8192, 32.0, True)
 LLAMA_70B = _llama(80, 8192, 64, 8, 128, 28672, 8.0, False)
 SHAPES = {"Llama-3.1-8B shape": LLAMA_8B, "Llama-3.2-1B shape": LLAMA_1B, "Llama-3.1-70B shape": LLAMA_70B}
-WORKLOADS = ("decode8b", "serve1b", "mixed70b", "sizes", "sizes1b", "prompts", "long", "widths", "portions", "tuvodra", "lilatar")
+WORKLOADS = ("decode8b", "serve1b", "mixed70b", "sizes", "sizes1b", "prompts", "long", "widths", "portions", "tuvodra", "lilatar", "vivisun")
 
 
 def flat_config(model: str, layers_run: int, global_batch: int, seq_len: int, page_size: int, **more) -> dict:
@@ -655,6 +657,45 @@ def run_lilatar(args) -> dict:
     return line
 
 
+def vivisun_shape(width, heads, kv_heads, dim, ff, kv_rank, layers, loop_times, vocab=128256):
+    """Layers in turns: attention with the Llama shape's heads (four taps on q, k and v, half of each head rotated with
+    bent frequencies, a gate) and latent attention with as many heads over one vector of `kv_rank` per token, each
+    with the Llama shape's feed-forward.  With loop_times > 1 the layers after the first run that often (then fewer
+    layers hold weights, the same number runs)."""
+    rot = {"dims": dim // 2, "base": 500000.0, "scaling": {"factor": 8.0, "original": 8192, "fast": 32.0, "slow": 1.0}}
+    two = [{"type": "attention", "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5, "conv": 4, "rot": rot},
+            "mlp": {"kind": "dense", "ff": ff}},
+           {"type": "latent_attention", "mixer": {"heads": heads, "dim": dim, "vdim": dim, "kv_rank": kv_rank, "scale": dim ** -0.5},
+            "mlp": {"kind": "dense", "ff": ff}}]
+    import copy
+    return {"architecture": "Vivisun", "vocab": vocab, "width": width, "norm": {"eps": 1e-6},
+            "layers": [copy.deepcopy(two[i % 2]) for i in range(layers)],
+            "loop": None if loop_times <= 1 else {"start": 1, "stop": layers, "times": loop_times}}
+
+
+def run_vivisun(args) -> dict:
+    """Prompt and decode throughput of the Vivisun decoder at two widths, each beside a Llama decoder of the same
+    width, heads, feed-forward and number of layer runs (random weights both)."""
+    runs = args.layers or 6
+    times = max(1, args.loop_times)
+    held = 1 + -(-(runs - 1) // times) if times > 1 else runs          # layers that hold weights
+    runs = 1 + (held - 1) * times if times > 1 else runs
+    sizes = {"1B widths": (LLAMA_1B, 2048, 32, 8, 64, 8192), "8B widths": (LLAMA_8B, 4096, 32, 8, 128, 14336)}
+    pairs = {size: {"vivisun": vivisun_shape(width, heads, kv_heads, dim, ff, args.kv_rank, held, times),
+                    "llama": dict(llama, num_hidden_layers=runs)}
+             for size, (llama, width, heads, kv_heads, dim, ff) in sizes.items()}
+    points = run_beside_llama(args, pairs, runs)
+    first = next(iter(points.values()))
+    line = base_line("decode_tokens_per_s", first["decode_tokens_per_s"], args.steps, args.warmup, first["decode_ms_per_step"] * 1e-3, args.dtype,
+                     {"model": "Vivisun (convolved, normed, half-rotated and gated attention in turns with latent attention with a sink; "
+                               "dynamic-tanh norms, both halves on the same stream) beside Llama of equal widths",
+                      "global_batch": args.batch, "seq_len": args.context, "parallelism": "single GPU", "layers_run": runs,
+                      "layers_with_weights": held, "loop_times": times, "kv_rank": args.kv_rank,
+                      "prefill_tokens": args.prefill_tokens, "page_size": 16})
+    line["points"] = points
+    return line
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -673,7 +714,9 @@ def main() -> int:
     ap.add_argument("--new-tokens", type=int, default=256, help="serve1b: tokens generated for each request")
     ap.add_argument("--max-batch-tokens", type=int, default=2048, help="serve1b: tokens a scheduler step may run")
     ap.add_argument("--window", type=int, default=1024, help="tuvodra, lilatar: keys an attention layer sees")
-    ap.add_argument("--only-size", default="", help="tuvodra, lilatar: run one of the sizes only (1B or 8B)")
+    ap.add_argument("--only-size", default="", help="tuvodra, lilatar, vivisun: run one of the sizes only (1B or 8B)")
+    ap.add_argument("--kv-rank", type=int, default=256, help="vivisun: width of the latent vector a token leaves in the cache")
+    ap.add_argument("--loop-times", type=int, default=1, help="vivisun: how often the layers after the first run in a row")
     ap.add_argument("--experts", type=int, default=16, help="lilatar: experts of a routed feed-forward")
     ap.add_argument("--top", type=int, default=4, help="lilatar: experts a token uses")
     ap.add_argument("--experts-by-rows-from", type=int, default=None,
@@ -686,7 +729,8 @@ def main() -> int:
     args.steps = args.steps if args.steps is not None else (8 if heavy else 64)
     args.warmup = args.warmup if args.warmup is not None else (2 if heavy else 8)
     line = {"decode8b": run_decode8b, "serve1b": run_serve1b, "mixed70b": run_mixed70b, "sizes": run_sizes, "sizes1b": run_sizes,
-            "prompts": run_prompts, "long": run_long, "widths": run_widths, "portions": run_portions, "tuvodra": run_tuvodra, "lilatar": run_lilatar}[args.workload](args)
+            "prompts": run_prompts, "long": run_long, "widths": run_widths, "portions": run_portions, "tuvodra": run_tuvodra, "lilatar": run_lilatar,
+            "vivisun": run_vivisun}[args.workload](args)
     from llm_rs_amd.kernels import kernels
     if kernels().times is not None:         # LLM_PERF: what was still to be shown of the per-kernel table
         kernels().times.dump()

@@ -21,11 +21,16 @@ struct AttnArgs {
     // sink[head], or null: the softmax's denominator of every query of the head also holds exp(sink[head]), once: a key
     // without a value, whose score is this number as it stands (not scaled, not bent, no penalty).
     const float* sink;
+    // gate, or null: 32-bit numbers [n_tokens, gate_stride], one for every gate_per consecutive output features of a
+    // token (1: a gate a feature; v_dim: a gate a head); the output is multiplied by their sigmoid, in 32-bit, before
+    // its one rounding.
+    const float* gate;
+    int gate_stride, gate_per;
 };
 // Whether a call is the plain one (values as wide as keys, no distance penalty, no soft cap, no kept first keys) that
 // every kernel file takes.
 static inline bool attn_is_plain(const AttnArgs& a) {
-    return a.v_dim == a.head_dim && a.dist_r1 == nullptr && a.softcap <= 0.0f && (a.keep_first <= 0 || a.window <= 0) && a.sink == nullptr;
+    return a.v_dim == a.head_dim && a.dist_r1 == nullptr && a.softcap <= 0.0f && (a.keep_first <= 0 || a.window <= 0) && a.sink == nullptr && a.gate == nullptr;
 }
 // The first key of the window of the query at `pos`, and how many of the first keys lie before it and stay visible.
 __host__ __device__ static inline int attn_window_lo(const AttnArgs& a, int pos) {
@@ -43,6 +48,12 @@ __device__ __forceinline__ float attn_sink_term(const AttnArgs& a, int head, flo
 }
 __device__ __forceinline__ float attn_sink_term_base2(const AttnArgs& a, int head, float m2) {
     return a.sink ? __builtin_amdgcn_exp2f(fmaf(a.sink[head], 1.4426950408889634f, -m2)) : 0.0f;
+}
+// What output feature d of `head` at `token` is multiplied by on its way out: the sigmoid of its gate, or 1.
+__device__ __forceinline__ float attn_gate(const AttnArgs& a, int token, int head, int d) {
+    if (a.gate == nullptr) return 1.0f;
+    float g = a.gate[(size_t)token * a.gate_stride + (head * a.v_dim + d) / a.gate_per];
+    return 1.0f / (1.0f + expf(-g));
 }
 // A step's entries bring their tokens as tiles of `per` tokens that never cross an entry; entries with one token
 // bring none when the caller splits those by key range instead.  Which entry holds tile `tile`, and which of that

@@ -171,7 +171,7 @@ __global__ __launch_bounds__(256) void attn_f32_tiles_kernel(const float* __rest
         for (int g = 0; g < 4; ++g) {
             f32x4 v;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) v[j] = O[dt][4 * g + j] * inv;
+            for (int j = 0; j < 4; ++j) v[j] = O[dt][4 * g + j] * inv * attn_gate(a, token, head, 4 * h + dt * 32 + 8 * g + j);
             *(f32x4*)(op + dt * 32 + 8 * g) = v;
         }
 }

@@ -109,7 +109,7 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
 #pragma unroll
     for (int i = 0; i < MAX_HEAD_DIM / 64; ++i) {
         int d = lane + 64 * i;
-        if (d < a.v_dim) orow[d] = from_f32<T>(acc[i] / l);
+        if (d < a.v_dim) orow[d] = from_f32<T>(acc[i] / l * attn_gate(a, t, h, d));
     }
 }
 
@@ -267,7 +267,7 @@ __global__ __launch_bounds__(64) void attention_generic_group_tokens_kernel(
 #pragma unroll
         for (int i = 0; i < NACC; ++i) {
             int d = lane + 64 * i;
-            if (d < a.v_dim) orow[d] = from_f32<T>(acc[g][i] / lg);
+            if (d < a.v_dim) orow[d] = from_f32<T>(acc[g][i] / lg * attn_gate(a, t, kvh * G + g, d));
         }
     }
 }
@@ -370,7 +370,7 @@ __global__ __launch_bounds__(64) void attention_generic_merge_kernel(
 #pragma unroll
     for (int i = 0; i < MAX_HEAD_DIM / 64; ++i) {
         int d = lane + 64 * i;
-        if (d < hd) orow[d] = from_f32<T>(o[i] / L);
+        if (d < hd) orow[d] = from_f32<T>(o[i] / L * attn_gate(a, t, h, d));
     }
 }
 
@@ -479,6 +479,7 @@ static int launch_generic(hipStream_t stream, const T* q, T* out, const T* k_cac
 // dist_r1, dist_r2: [n_heads] 32-bit, the logarithmic distance penalty of AttnArgs, or both null.
 // softcap, keep_first: the soft cap of the scores and the first keys that a window keeps (AttnArgs), or 0.
 // sink: [n_heads] 32-bit, a number a head that the softmax's denominator also holds the exponential of, or null.
+// gate: [n_tokens, gate_stride] 32-bit, one number for every gate_per output features, whose sigmoid they are multiplied by, or null.
 extern "C" int llmrs_attention_ext(hipStream_t stream, int dtype, const void* q, int q_stride, void* out, int out_stride,
                                    const void* k_cache, const void* v_cache, const int* block_table, int table_width,
                                    const int* token_entry, const int* positions, const int* q_starts,
@@ -486,7 +487,7 @@ extern "C" int llmrs_attention_ext(hipStream_t stream, int dtype, const void* q,
                                    int head_dim, int page_size, int num_pages, int window, float scale,
                                    void* scratch, size_t scratch_bytes, int max_seq_len, int n_single, long single_keys,
                                    int allow_mfma, int v_dim, const float* dist_r1, const float* dist_r2, float softcap,
-                                   int keep_first, const float* sink) {
+                                   int keep_first, const float* sink, const float* gate, int gate_stride, int gate_per) {
     LLMRS_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && head_dim > 0 && v_dim > 0, "attention: bad sizes");
     LLMRS_REQUIRE(v_dim <= MAX_HEAD_DIM, "attention: value width %d exceeds %d", v_dim, MAX_HEAD_DIM);
     LLMRS_REQUIRE((dist_r1 == nullptr) == (dist_r2 == nullptr), "attention: the distance penalty needs both of its tables");
@@ -497,12 +498,14 @@ extern "C" int llmrs_attention_ext(hipStream_t stream, int dtype, const void* q,
     LLMRS_REQUIRE(window >= 0, "attention: negative window");
     LLMRS_REQUIRE(softcap >= 0.0f && keep_first >= 0, "attention: negative soft cap or number of kept first keys");
     LLMRS_REQUIRE(n_heads <= 65535, "attention: too many heads for one launch");
+    LLMRS_REQUIRE(gate == nullptr || (gate_per > 0 && (n_heads * v_dim) % gate_per == 0 && gate_stride >= n_heads * v_dim / gate_per),
+                  "attention: a gate for every %d of %d output features at rows of %d does not fit", gate_per, n_heads * v_dim, gate_stride);
     LLMRS_REQUIRE(n_single <= n_entries, "attention: %d single-token entries among %d entries", n_single, n_entries);
     LLMRS_REQUIRE(n_single != n_entries || n_tokens == n_entries,
                   "attention: every entry is said to bring one token, but %d entries bring %d tokens", n_entries, n_tokens);
     if (n_tokens == 0) return 0;
     AttnArgs a{n_tokens, n_heads, n_kv_heads, head_dim, page_size, table_width, num_pages, q_stride, out_stride, window, scale,
-               v_dim, dist_r1, dist_r2, softcap, window > 0 ? keep_first : 0, sink};
+               v_dim, dist_r1, dist_r2, softcap, window > 0 ? keep_first : 0, sink, gate, gate_stride, gate_per};
     if (dtype == LLMRS_BF16 && allow_mfma) {
         int took = llmrs_attention_bf16_mfma(stream, (const bf16*)q, (bf16*)out, (const bf16*)k_cache, (const bf16*)v_cache,
                                              block_table, token_entry, positions, q_starts, seq_lens, n_entries,
@@ -535,5 +538,5 @@ extern "C" int llmrs_attention(hipStream_t stream, int dtype, const void* q, int
     return llmrs_attention_ext(stream, dtype, q, q_stride, out, out_stride, k_cache, v_cache, block_table, table_width,
                                token_entry, positions, q_starts, seq_lens, n_entries, n_tokens, n_heads, n_kv_heads,
                                head_dim, page_size, num_pages, window, scale, scratch, scratch_bytes, max_seq_len, n_single,
-                               single_keys, allow_mfma, head_dim, nullptr, nullptr, 0.0f, 0, nullptr);
+                               single_keys, allow_mfma, head_dim, nullptr, nullptr, 0.0f, 0, nullptr, nullptr, 0, 1);
 }

@@ -295,7 +295,7 @@ __global__ __launch_bounds__(256) void attn_tiles_kernel(const bf16* __restrict_
         for (int i4 = 0; i4 < 4; ++i4) {
             bf16x4 v;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) v[j] = (bf16)(O[dt][i4 * 4 + j] * inv);
+            for (int j = 0; j < 4; ++j) v[j] = (bf16)(O[dt][i4 * 4 + j] * inv * attn_gate(a, token, head, o_feature(dt, i4 * 4, h) + j));
             *(bf16x4*)(op + o_feature(dt, i4 * 4, h)) = v;
         }
 }
@@ -560,7 +560,7 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(HD <
         for (int i4 = 0; i4 < 4; ++i4) {
             bf16x4 v;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) v[j] = (bf16)(O[dt][i4 * 4 + j] * inv);
+            for (int j = 0; j < 4; ++j) v[j] = (bf16)(O[dt][i4 * 4 + j] * inv * attn_gate(a, token, head, o_feature(dt, i4 * 4, h) + j));
             *(bf16x4*)(op + o_feature(dt, i4 * 4, h)) = v;
         }
 }
@@ -923,7 +923,7 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(const float* __restrict
         for (int c = 0; c < AHEAD; ++c)
             if (ch + c < n_chunks) o = fmaf(v[c], weight[ch + c], o);
     }
-    out[(size_t)token * a.out_stride + (size_t)head * hd + d] = (bf16)(o / (L + attn_sink_term_base2(a, head, M)));
+    out[(size_t)token * a.out_stride + (size_t)head * hd + d] = (bf16)(o / (L + attn_sink_term_base2(a, head, M)) * attn_gate(a, token, head, d));
 }
 
 // The merge for more than a few chunks (131,000 keys of one request are 256 chunks of 512).  One thread per
@@ -1005,7 +1005,7 @@ __global__ __launch_bounds__(MERGE_GROUP_THREADS) void attn_merge_groups_kernel(
     if (tid < hd) {
         float o = 0.0f;
         for (int k = 0; k < groups; ++k) o += sums[k * hd + tid];
-        out[(size_t)token * a.out_stride + (size_t)head * hd + tid] = (bf16)(o / (L + attn_sink_term_base2(a, head, M)));
+        out[(size_t)token * a.out_stride + (size_t)head * hd + tid] = (bf16)(o / (L + attn_sink_term_base2(a, head, M)) * attn_gate(a, token, head, tid));
     }
 }
 

@@ -66,7 +66,8 @@ extern "C" int llmrs_latent_finish(hipStream_t stream, int dtype, const float* s
 
 // ---- every head by its own matrix -----------------------------------------------------------------------------------
 // A block of 256 threads makes 64 tokens x 64 outputs of one head: 16 inputs at a time through LDS, every thread a
-// 4 x 4 corner in 32-bit multiply-adds (any sizes, any type).
+// 4 x 4 corner in 32-bit multiply-adds (any sizes, any type; what 32-bit runs use, and bfloat16 at sizes the matrix-core
+// kernel below does not take).
 #define HP_TILE 64
 #define HP_K 16
 template <class T>
@@ -113,6 +114,79 @@ __global__ __launch_bounds__(256) void head_product_kernel(const T* __restrict__
     }
 }
 
+// The same on the matrix cores, for bfloat16 with rows of whole 16-byte pieces: a wave makes MT x NT tiles of 16 tokens
+// x 16 outputs with v_mfma_f32_16x16x32_bf16, its operands straight from memory (a head's matrix and a tile's rows are
+// small and stay in the caches; 32 inputs a turn, lane (row, g) brings inputs 8g .. 8g + 7 of its row).  The four waves
+// of a block lie along the tokens, or (ALONG_N, steps of few rows) along the outputs.  Every output's sum runs over
+// the inputs in the same order whatever the tiling, so a row's result does not depend on what else is in the step.
+typedef __bf16 hp_bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 hp_bf16x4 __attribute__((ext_vector_type(4)));
+typedef float hp_f32x4 __attribute__((ext_vector_type(4)));
+
+template <int MT, int NT, bool ALONG_N>
+__global__ __launch_bounds__(256) void head_product_mfma_kernel(const bf16* __restrict__ a, int lda, const bf16* __restrict__ w,
+                                                                bf16* __restrict__ out, int ldo, int n_tokens, int n_in, int n_out,
+                                                                const float* __restrict__ gate, int ldg, int wide_stores) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, row = lane & 15, g = lane >> 4;
+    const int h = blockIdx.z;
+    const int m0 = (ALONG_N ? blockIdx.y : blockIdx.y * 4 + wave) * (MT * 16);
+    const int n0 = (ALONG_N ? blockIdx.x * 4 + wave : blockIdx.x) * (NT * 16);
+    if (m0 >= n_tokens || n0 >= n_out) return;
+    const bf16* xp[MT];
+    const bf16* wp[NT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) xp[mt] = a + (size_t)min(m0 + mt * 16 + row, n_tokens - 1) * lda + (size_t)h * n_in;
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) wp[nt] = w + ((size_t)h * n_out + min(n0 + nt * 16 + row, n_out - 1)) * n_in;
+    hp_f32x4 acc[MT][NT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = hp_f32x4{0.f, 0.f, 0.f, 0.f};
+    const hp_bf16x8 zero = {};
+#pragma unroll 2
+    for (int k0 = 0; k0 < n_in; k0 += 32) {
+        int k = k0 + 8 * g;
+        bool in = k < n_in;                     // (rows are whole pieces of 8: a piece is inside or outside)
+        hp_bf16x8 x[MT], ww[NT];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) x[mt] = in ? *(const hp_bf16x8*)(xp[mt] + k) : zero;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) ww[nt] = in ? *(const hp_bf16x8*)(wp[nt] + k) : zero;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ww[nt], x[mt], acc[mt][nt], 0, 0, 0);
+    }
+    // the lane holds, of tile (mt, nt), token m0 + 16 mt + row and outputs n0 + 16 nt + 4 g .. + 3
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        int m = m0 + mt * 16 + row;
+        if (m >= n_tokens) continue;
+        float gm = gate ? 1.0f / (1.0f + expf(-gate[(size_t)m * ldg + h])) : 1.0f;
+        bf16* dst = out + (size_t)m * ldo + (size_t)h * n_out;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            int n = n0 + nt * 16 + 4 * g;
+            if (wide_stores && n + 3 < n_out) {
+                *(hp_bf16x4*)(dst + n) = hp_bf16x4{(bf16)(acc[mt][nt][0] * gm), (bf16)(acc[mt][nt][1] * gm),
+                                                   (bf16)(acc[mt][nt][2] * gm), (bf16)(acc[mt][nt][3] * gm)};
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    if (n + r < n_out) dst[n + r] = (bf16)(acc[mt][nt][r] * gm);
+            }
+        }
+    }
+}
+
+template <int MT, int NT, bool ALONG_N>
+static void launch_head_product_mfma(hipStream_t stream, const bf16* a, int lda, const bf16* w, bf16* out, int ldo, int n_tokens,
+                                     int heads, int n_in, int n_out, const float* gate, int ldg, int wide_stores) {
+    dim3 grid(ceil_div(n_out, NT * 16 * (ALONG_N ? 4 : 1)), ceil_div(n_tokens, MT * 16 * (ALONG_N ? 1 : 4)), heads);
+    head_product_mfma_kernel<MT, NT, ALONG_N><<<grid, 256, 0, stream>>>(a, lda, w, out, ldo, n_tokens, n_in, n_out, gate, ldg, wide_stores);
+}
+
 // a: [n_tokens, lda], head h's inputs at columns h * n_in ..; w: [heads][n_out][n_in]; out: [n_tokens, ldo], head h's
 // outputs at columns h * n_out ..; all in `dtype`, sums in 32-bit.  gate: [n_tokens, ldg] 32-bit, a column a head, or null.
 extern "C" int llmrs_head_product(hipStream_t stream, int dtype, const void* a, int lda, const void* w, void* out, int ldo,
@@ -122,7 +196,18 @@ extern "C" int llmrs_head_product(hipStream_t stream, int dtype, const void* a, 
     LLMRS_REQUIRE(heads <= 65535 && ceil_div(n_tokens, HP_TILE) <= 65535, "head_product: too many heads or tokens for one launch");
     LLMRS_REQUIRE(dtype == LLMRS_F32 || dtype == LLMRS_BF16, "head_product: unknown dtype %d", dtype);
     if (n_tokens == 0) return 0;
-    (void)allow_mfma;
+    auto pieces = [](const void* p, int ld) { return ((uintptr_t)p & 15) == 0 && ld % 8 == 0; };
+    if (dtype == LLMRS_BF16 && allow_mfma && n_in % 8 == 0 && pieces(a, lda) && pieces(w, n_in) &&
+        ceil_div(n_tokens, 16) <= 65535) {
+        int wide = ((uintptr_t)out & 7) == 0 && ldo % 4 == 0 && n_out % 4 == 0;
+        const bf16 *ab = (const bf16*)a, *wb = (const bf16*)w;
+        bf16* ob = (bf16*)out;
+        if (n_tokens <= 16) launch_head_product_mfma<1, 1, true>(stream, ab, lda, wb, ob, ldo, n_tokens, heads, n_in, n_out, gate, ldg, wide);
+        else if (n_tokens <= 512) launch_head_product_mfma<1, 4, false>(stream, ab, lda, wb, ob, ldo, n_tokens, heads, n_in, n_out, gate, ldg, wide);
+        else launch_head_product_mfma<4, 4, false>(stream, ab, lda, wb, ob, ldo, n_tokens, heads, n_in, n_out, gate, ldg, wide);
+        LLMRS_LAUNCH_CHECK("head_product");
+        return 0;
+    }
     dim3 grid(ceil_div(n_out, HP_TILE), ceil_div(n_tokens, HP_TILE), heads);
     if (dtype == LLMRS_F32)
         head_product_kernel<float><<<grid, 256, 0, stream>>>((const float*)a, lda, (const float*)w, (float*)out, ldo, n_tokens, n_in, n_out, gate, ldg);

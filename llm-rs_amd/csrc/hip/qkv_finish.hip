@@ -32,14 +32,16 @@ struct QkvFinishArgs {
     const int* token_entry;
 };
 
-// One wave for each (token, head of q, k or v).
+// One wave for each (token, head of q, k or v); a block's four waves take four neighbouring tokens of the same head
+// (a quarter of the blocks to hand out, and the rows that a convolution reads again lie in the same block's reach).
 template <class T>
-__global__ __launch_bounds__(64) void qkv_finish_kernel(const float* __restrict__ sums, const float* __restrict__ bias,
+__global__ __launch_bounds__(256) void qkv_finish_kernel(const float* __restrict__ sums, const float* __restrict__ bias,
                                                          T* __restrict__ q, const int* __restrict__ slot_map,
                                                          T* __restrict__ k_cache, T* __restrict__ v_cache,
                                                          const int* __restrict__ positions, const float* __restrict__ inv_freq,
                                                          QkvFinishArgs a) {
-    int t = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+    int t = blockIdx.x * 4 + (threadIdx.x >> 6), head = blockIdx.y, lane = threadIdx.x & 63;
+    if (t >= a.n_tokens) return;
     bool is_q = head < a.n_heads, is_k = !is_q && head < a.n_heads + a.n_kv_heads;
     if (!is_q && !a.write_kv) return;
     int width = (is_q || is_k) ? a.head_dim : a.v_dim;
@@ -163,11 +165,11 @@ extern "C" int llmrs_qkv_finish(hipStream_t stream, int dtype, const float* sums
     if (n_tokens == 0) return 0;
     QkvFinishArgs a{n_tokens, n_heads, n_kv_heads, head_dim, v_dim, in_stride, q_stride, page_size, num_pages, write_kv, eps, rotary_dim,
                     gain, q_weight, k_weight, taps, n_taps, columns, state, state_stride, q_starts, slots, token_entry};
-    dim3 grid(n_tokens, n_heads + 2 * n_kv_heads);
+    dim3 grid(ceil_div(n_tokens, 4), n_heads + 2 * n_kv_heads);
     if (dtype == LLMRS_F32)
-        qkv_finish_kernel<float><<<grid, 64, 0, stream>>>(sums, bias, (float*)q, slot_map, (float*)k_cache, (float*)v_cache, positions, inv_freq, a);
+        qkv_finish_kernel<float><<<grid, 256, 0, stream>>>(sums, bias, (float*)q, slot_map, (float*)k_cache, (float*)v_cache, positions, inv_freq, a);
     else if (dtype == LLMRS_BF16)
-        qkv_finish_kernel<bf16><<<grid, 64, 0, stream>>>(sums, bias, (bf16*)q, slot_map, (bf16*)k_cache, (bf16*)v_cache, positions, inv_freq, a);
+        qkv_finish_kernel<bf16><<<grid, 256, 0, stream>>>(sums, bias, (bf16*)q, slot_map, (bf16*)k_cache, (bf16*)v_cache, positions, inv_freq, a);
     else
         return llmrs_fail("qkv_finish: unknown dtype %d", dtype);
     LLMRS_LAUNCH_CHECK("qkv_finish");

@@ -194,7 +194,7 @@ class HipKernels(Kernels):
             "llmrs_argmax_rows": [V, V, I, I, I, V, V, c_size_t],
             "llmrs_sample_rows": [V, V, I, I, I, V, V],
             "llmrs_place_ids": [V, V, I, V, V, V, I, I, I],
-            "llmrs_attention_ext": [V, I, V, I, V, I, V, V, V, I, V, V, V, V, I, I, I, I, I, I, I, I, F, V, c_size_t, I, I, ctypes.c_long, I, I, V, V, F, I, V],
+            "llmrs_attention_ext": [V, I, V, I, V, I, V, V, V, I, V, V, V, V, I, I, I, I, I, I, I, I, F, V, c_size_t, I, I, ctypes.c_long, I, I, V, V, F, I, V, V, I, I],
             "llmrs_group_rmsnorm": [V, I, V, V, ctypes.c_long, I, V, V, V, I, I, I, F, V, V, V, V, V],
             "llmrs_streams_mix": [V, V, ctypes.c_long, I, V, V, V, ctypes.c_long],
             "llmrs_streams_copy_first": [V, V, ctypes.c_long, I, ctypes.c_long],
@@ -486,8 +486,10 @@ class HipKernels(Kernels):
 
     def attention(self, q, out, k_cache, v_cache, block_table, token_entry, positions, q_starts, seq_lens,
                   n_heads, n_kv_heads, head_dim, page_size, num_pages, window, scale, scratch=None, max_seq_len=0, n_single=-1,
-                  single_keys=0, value_dim=0, distance=None, softcap=0.0, keep_first=0, sink=None) -> None:
-        """sink: float32 [n_heads] or None: the softmax's denominator of head h also holds exp(sink[h]), once for every
+                  single_keys=0, value_dim=0, distance=None, softcap=0.0, keep_first=0, sink=None, gate=None, gate_per=1) -> None:
+        """gate: float32 [T, n_heads * value_dim / gate_per] or None: every gate_per consecutive output features of a token
+        are multiplied by the sigmoid of their number (32-bit, before the one rounding).
+        sink: float32 [n_heads] or None: the softmax's denominator of head h also holds exp(sink[h]), once for every
         query (a key without a value; not scaled).  single_keys: how many keys the single-token entries see together (windows counted), 0 if unknown.
         value_dim: the width of a value where it is not a key's (0: the same).  distance: (r1, r2), float32 [n_heads]
         each: r1[h] * ln(1 + r2[h] * (i - j)) is taken off the scaled score of query i and key j.  softcap > 0: the
@@ -497,10 +499,10 @@ class HipKernels(Kernels):
         assert block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous()
         v_dim = int(value_dim) or head_dim
         assert k_cache.numel() == num_pages * n_kv_heads * page_size * head_dim and v_cache.numel() == num_pages * n_kv_heads * page_size * v_dim
-        if v_dim != head_dim or distance is not None or softcap > 0 or (keep_first > 0 and window > 0) or sink is not None:
+        if v_dim != head_dim or distance is not None or softcap > 0 or (keep_first > 0 and window > 0) or sink is not None or gate is not None:
             return self._attention_ext(q, out, k_cache, v_cache, block_table, token_entry, positions, q_starts, seq_lens, n_heads,
                                        n_kv_heads, head_dim, page_size, num_pages, window, scale, scratch, max_seq_len, n_single,
-                                       single_keys, v_dim, distance, softcap, keep_first, sink)
+                                       single_keys, v_dim, distance, softcap, keep_first, sink, gate, gate_per)
         T = q.shape[0]
         assert token_entry.shape[0] == T and positions.shape[0] == T and out.shape[0] == T
         moved = flops = 0
@@ -519,8 +521,10 @@ class HipKernels(Kernels):
 
     def _attention_ext(self, q, out, k_cache, v_cache, block_table, token_entry, positions, q_starts, seq_lens, n_heads,
                        n_kv_heads, head_dim, page_size, num_pages, window, scale, scratch, max_seq_len, n_single, single_keys,
-                       v_dim, distance, softcap=0.0, keep_first=0, sink=None) -> None:
+                       v_dim, distance, softcap=0.0, keep_first=0, sink=None, gate=None, gate_per=1) -> None:
         T = q.shape[0]
+        assert gate is None or (gate.dtype == torch.float32 and gate.stride(1) == 1 and gate.shape[0] == T and gate_per >= 1
+                                and (n_heads * v_dim) % gate_per == 0 and gate.shape[1] == n_heads * v_dim // gate_per)
         assert sink is None or (sink.dtype == torch.float32 and sink.numel() == n_heads and sink.is_contiguous())
         assert token_entry.shape[0] == T and positions.shape[0] == T and out.shape[0] == T
         r1 = r2 = None
@@ -539,7 +543,8 @@ class HipKernels(Kernels):
                   _p(block_table), block_table.shape[1], _p(token_entry), _p(positions), _p(q_starts), _p(seq_lens),
                   block_table.shape[0], T, n_heads, n_kv_heads, head_dim, page_size, num_pages, window, scale,
                   _p(scratch), 0 if scratch is None else scratch.numel() * scratch.element_size(), int(max_seq_len),
-                  int(n_single), int(single_keys), int(self.allow_mfma), v_dim, _p(r1), _p(r2), float(softcap), int(keep_first), _p(sink))
+                  int(n_single), int(single_keys), int(self.allow_mfma), v_dim, _p(r1), _p(r2), float(softcap), int(keep_first), _p(sink),
+                  _p(gate), 0 if gate is None else gate.stride(0), int(gate_per))
 
     # out[i, :] = weight * groupnorm(sum_s w_in[s] * x[s][rows[i] or i, :]); x: [T, D] or [S, T, D] float32
     def group_rmsnorm(self, out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, eps: float, groups: int,

@@ -256,7 +256,8 @@ class Attention(KeyedBySplitChunk, Mixer):
 
     def _forward_prepared(self, ctx, x, h, cache):
         """The product's 32-bit sums -> convolution, biases, norm and rotation of q and k, cache write -> attention with
-        the distance penalty, the soft cap and the kept first keys -> the output gate -> the output projection."""
+        the distance penalty, the soft cap, the kept first keys and the output gate (applied to the 32-bit results on their
+        way out) -> the output projection."""
         k = kernels()
         T = x.shape[0]
         conv_state = None
@@ -285,9 +286,8 @@ class Attention(KeyedBySplitChunk, Mixer):
         k.attention(q, o, cache.k, cache.v, ctx.block_tables[g], ctx.token_entry, ctx.positions, ctx.q_starts, ctx.seq_lens,
                     self.heads, self.kv_heads, self.head_dim, cache.page_size, cache.num_pages, self.window, self.scale,
                     scratch, ctx.max_seq_len, ctx.n_single, self._keys_for_the_split(ctx), value_dim=self.value_dim,
-                    distance=None if self.distance is None else (self.r1, self.r2), softcap=self.softcap, keep_first=self.keep_first)
-        if self.gate is not None:
-            k.sigmoid_gate(o, sums[:, self.qkv_width:], 1 if self.gate == "feature" else self.value_dim)
+                    distance=None if self.distance is None else (self.r1, self.r2), softcap=self.softcap, keep_first=self.keep_first,
+                    gate=sums[:, self.qkv_width:] if self.gate is not None else None, gate_per=1 if self.gate == "feature" else self.value_dim)
         k.gemm(o, self.w_o, h, EPI_ACCUM_F32, ctx.gemm_workspace(o, self.w_o))
         if self.has_o_bias and not self.output_bias_left_to_holder:
             k.add_bias_rows(h, self.o_bias)

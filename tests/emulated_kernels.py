@@ -147,7 +147,7 @@ class EmulatedKernels(Kernels):
 
     def attention(self, q, out, k_cache, v_cache, block_table, token_entry, positions, q_starts, seq_lens,
                   n_heads, n_kv_heads, head_dim, page_size, num_pages, window, scale, scratch=None, max_seq_len=0, n_single=-1,
-                  single_keys=0, value_dim=0, distance=None, softcap=0.0, keep_first=0, sink=None):
+                  single_keys=0, value_dim=0, distance=None, softcap=0.0, keep_first=0, sink=None, gate=None, gate_per=1):
         T = q.shape[0]
         v_dim = value_dim or head_dim
         kc = k_cache.view(num_pages, n_kv_heads, page_size, head_dim).float()
@@ -174,7 +174,11 @@ class EmulatedKernels(Kernels):
                     p = torch.softmax(torch.cat([s, sink[h:h + 1]]), dim=0)[:-1]
                 else:
                     p = torch.softmax(s, dim=0)
-                out[t, h * v_dim:(h + 1) * v_dim] = (p @ vals[:, g, :]).to(out.dtype)
+                o = p @ vals[:, g, :]
+                if gate is not None:         # a number for every gate_per output features: they are multiplied by its sigmoid
+                    cols = torch.arange(h * v_dim, (h + 1) * v_dim) // gate_per
+                    o = o * (1.0 / (1.0 + torch.exp(-gate[t, cols].float())))
+                out[t, h * v_dim:(h + 1) * v_dim] = o.to(out.dtype)
 
     def group_rmsnorm(self, out, x, weight, eps, groups, rows=None, w_in=None, zero=None, combined=None, mix=None):
         assert x.dim() == 2 and w_in is None and combined is None and mix is None, "one stream only"

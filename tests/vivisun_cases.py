@@ -64,10 +64,21 @@ def one_layer(layer, width=40, vocab=61, loop=None):
     return config(width, vocab, [layer], loop)
 
 
+def loud(tensors) -> None:
+    """Random weights under which tokens differ: a dynamic tanh does not bring small embeddings up to size as a norm that
+    divides would (its bias would be all that the layers see), so the token table is of order one; queries and the
+    mixers' outputs are enlarged so that scores spread and what a mixer says counts beside the stream."""
+    for name in list(tensors):
+        factor = 50.0 if name == "embed" else 8.0 if name.endswith(".mix.q") else 4.0 if name.endswith(".mix.o") else None
+        if factor is not None:
+            tensors[name] = (tensors[name].double() * factor).to(tensors[name].dtype)
+
+
 def make_model(cfg: dict, seed: int = 0, change=None):
     """(typed config, {name: bfloat16 tensor}); `change(tensors)` may put values of its own in."""
     typed = VivisunConfig.from_dict(cfg)
     tensors = random_model_tensors(typed, seed)
+    loud(tensors)
     if change is not None:
         change(tensors)
     return typed, tensors
