@@ -34,7 +34,8 @@ struct QkvFinishArgs {
 
 // One wave for each (token, head of q, k or v); a block's four waves take four neighbouring tokens of the same head
 // (a quarter of the blocks to hand out, and the rows that a convolution reads again lie in the same block's reach).
-template <class T>
+// NI: how many features a lane holds (heads of up to 64 NI features), so that narrow heads pay for no empty turns.
+template <class T, int NI>
 __global__ __launch_bounds__(256) void qkv_finish_kernel(const float* __restrict__ sums, const float* __restrict__ bias,
                                                          T* __restrict__ q, const int* __restrict__ slot_map,
                                                          T* __restrict__ k_cache, T* __restrict__ v_cache,
@@ -49,14 +50,27 @@ __global__ __launch_bounds__(256) void qkv_finish_kernel(const float* __restrict
                    : is_k ? a.n_heads * a.head_dim + (head - a.n_heads) * a.head_dim
                           : (a.n_heads + a.n_kv_heads) * a.head_dim + (head - a.n_heads - a.n_kv_heads) * a.v_dim;
     const float* src = sums + (size_t)t * a.in_stride + col;
-    float x[8];            // features lane, lane + 64, ... (heads of up to 512)
+    float x[NI];           // features lane, lane + 64, ... (heads of up to 512)
     float ss = 0.0f;
+    // what the later stages read from memory is asked for now, beside the rows: a step of few tokens is a chain of
+    // trips to memory, and these do not depend on one another
+    const bool normed = (is_q || is_k) && a.eps > 0.0f, turned = (is_q || is_k) && a.rotary_dim > 0;
+    const float* nw = is_q ? a.q_weight : a.k_weight;
+    float nwv[NI], freq[NI];
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+        int d = lane + 64 * i;
+        nwv[i] = (normed && nw && d < width) ? nw[d] : 1.0f;
+        freq[i] = (turned && d < a.rotary_dim) ? inv_freq[d >> 1] : 0.0f;
+    }
+    const float pos = turned ? (float)positions[t] : 0.0f;
+    const int slot = is_q ? 0 : slot_map[t];
     if (a.taps) {
         int e = a.token_entry[t];
         int place = t - a.q_starts[e];                     // the token's place in its entry
         const float* sp = a.n_taps > 1 ? a.state + (size_t)a.slots[e] * a.state_stride + col : nullptr;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
+        for (int i = 0; i < NI; ++i) {
             int d = lane + 64 * i;
             float acc = 0.0f;
             if (d < width) {
@@ -73,36 +87,34 @@ __global__ __launch_bounds__(256) void qkv_finish_kernel(const float* __restrict
         }
     } else {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
+        for (int i = 0; i < NI; ++i) {
             int d = lane + 64 * i;
             x[i] = d < width ? src[d] + (bias ? bias[col + d] : 0.0f) : 0.0f;
             ss = fmaf(x[i], x[i], ss);
         }
     }
     float inv = 1.0f;
-    if ((is_q || is_k) && a.eps > 0.0f) {
+    if (normed) {
         inv = 1.0f / sqrtf(wave_sum(ss) / (float)width + a.eps);
-        const float* nw = is_q ? a.q_weight : a.k_weight;
         if (nw) {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
+            for (int i = 0; i < NI; ++i) {
                 int d = lane + 64 * i;
-                x[i] = d < width ? x[i] * inv * nw[d] : 0.0f;
+                x[i] = d < width ? x[i] * inv * nwv[i] : 0.0f;
             }
             inv = 1.0f;
         }
     }
-    if ((is_q || is_k) && a.rotary_dim > 0) {
+    if (turned) {
         // feature d's partner d ^ 1 lies in the neighbouring lane; angles and the turn in 32-bit
-        float pos = (float)positions[t];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
+        for (int i = 0; i < NI; ++i) {
             int d = lane + 64 * i;
             x[i] *= inv;
             float other = __shfl_xor(x[i], 1, 64);
             if (d < a.rotary_dim) {
                 float s, c;
-                sincosf(pos * inv_freq[d >> 1], &s, &c);
+                sincosf(pos * freq[i], &s, &c);
                 s *= a.gain;
                 c *= a.gain;
                 x[i] = (d & 1) ? fmaf(x[i], c, other * s) : fmaf(x[i], c, -other * s);
@@ -113,17 +125,16 @@ __global__ __launch_bounds__(256) void qkv_finish_kernel(const float* __restrict
     if (is_q) {
         T* dst = q + (size_t)t * a.q_stride + col;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
+        for (int i = 0; i < NI; ++i) {
             int d = lane + 64 * i;
             if (d < width) dst[d] = from_f32<T>(x[i] * inv);
         }
         return;
     }
-    int slot = slot_map[t];
     if (slot < 0 || slot >= a.num_pages * a.page_size) return;  // never write outside the cache
     int page = slot / a.page_size, off = slot % a.page_size;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < NI; ++i) {
         int d = lane + 64 * i;
         if (d >= width) continue;
         if (is_k)
@@ -166,12 +177,14 @@ extern "C" int llmrs_qkv_finish(hipStream_t stream, int dtype, const float* sums
     QkvFinishArgs a{n_tokens, n_heads, n_kv_heads, head_dim, v_dim, in_stride, q_stride, page_size, num_pages, write_kv, eps, rotary_dim,
                     gain, q_weight, k_weight, taps, n_taps, columns, state, state_stride, q_starts, slots, token_entry};
     dim3 grid(ceil_div(n_tokens, 4), n_heads + 2 * n_kv_heads);
-    if (dtype == LLMRS_F32)
-        qkv_finish_kernel<float><<<grid, 256, 0, stream>>>(sums, bias, (float*)q, slot_map, (float*)k_cache, (float*)v_cache, positions, inv_freq, a);
-    else if (dtype == LLMRS_BF16)
-        qkv_finish_kernel<bf16><<<grid, 256, 0, stream>>>(sums, bias, (bf16*)q, slot_map, (bf16*)k_cache, (bf16*)v_cache, positions, inv_freq, a);
-    else
-        return llmrs_fail("qkv_finish: unknown dtype %d", dtype);
+    int widest = head_dim > v_dim ? head_dim : v_dim;
+    if (dtype != LLMRS_F32 && dtype != LLMRS_BF16) return llmrs_fail("qkv_finish: unknown dtype %d", dtype);
+#define QKV_FINISH(T, NI) qkv_finish_kernel<T, NI><<<grid, 256, 0, stream>>>(sums, bias, (T*)q, slot_map, (T*)k_cache, (T*)v_cache, positions, inv_freq, a)
+#define QKV_FINISH_BY_WIDTH(T) do { if (widest <= 64) QKV_FINISH(T, 1); else if (widest <= 128) QKV_FINISH(T, 2); \
+                                     else if (widest <= 256) QKV_FINISH(T, 4); else QKV_FINISH(T, 8); } while (0)
+    if (dtype == LLMRS_F32) QKV_FINISH_BY_WIDTH(float); else QKV_FINISH_BY_WIDTH(bf16);
+#undef QKV_FINISH_BY_WIDTH
+#undef QKV_FINISH
     LLMRS_LAUNCH_CHECK("qkv_finish");
     return 0;
 }
