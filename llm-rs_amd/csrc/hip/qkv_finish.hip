@@ -144,6 +144,164 @@ __global__ __launch_bounds__(256) void qkv_finish_kernel(const float* __restrict
     }
 }
 
+// The same with four neighbouring columns a lane, for heads whose width is a power of two from 8 to 256 and rows of whole
+// 16-byte pieces: a wave takes 256 columns of a token (several heads, whatever they are heads of) and four tokens one after
+// the other, a block sixteen tokens, whose rows a convolution finds in LDS; every load is 16 bytes; a head's sum of squares is added up within its own head_dim / 4 lanes; the two
+// partners of a rotation lie in the same lane.  Which of the two kernels runs depends on the sizes and the rows'
+// alignment alone, never on what a step holds.
+template <class T>
+__device__ __forceinline__ void qkv_store4(T* dst, const float (&v)[4]);
+template <>
+__device__ __forceinline__ void qkv_store4<float>(float* dst, const float (&v)[4]) {
+    *(float4*)dst = float4{v[0], v[1], v[2], v[3]};
+}
+template <>
+__device__ __forceinline__ void qkv_store4<bf16>(bf16* dst, const float (&v)[4]) {
+    typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+    *(bf16x4_t*)dst = bf16x4_t{(bf16)v[0], (bf16)v[1], (bf16)v[2], (bf16)v[3]};
+}
+
+// TPW: tokens a wave takes, one after the other (a block takes 4 TPW): four over many rows, one in steps of few rows,
+// which are a chain of trips to memory; the sums are the same bits either way.
+template <class T, int TPW>
+__global__ __launch_bounds__(256) void qkv_finish_wide_kernel(const float* __restrict__ sums, const float* __restrict__ bias,
+                                                              T* __restrict__ q, const int* __restrict__ slot_map,
+                                                              T* __restrict__ k_cache, T* __restrict__ v_cache,
+                                                              const int* __restrict__ positions, const float* __restrict__ inv_freq,
+                                                              QkvFinishArgs a) {
+    // With taps: the block's rows of its 256 columns, and the n_taps - 1 rows before them, once through LDS (a row is
+    // read by up to n_taps tokens): [4 TPW + n_taps - 1][64 lanes] pieces of four columns.
+    extern __shared__ float4 staged[];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    constexpr int QKV_WIDE_TOKENS = 4 * TPW;
+    const int t0 = blockIdx.x * QKV_WIDE_TOKENS;
+    const int c = blockIdx.y * 256 + 4 * lane;                 // this lane's first column
+    const int q_cols = a.n_heads * a.head_dim, qk_cols = q_cols + a.n_kv_heads * a.head_dim;
+    const bool inside = c < a.columns, is_q = c < q_cols, is_k = !is_q && c < qk_cols, is_v = inside && !is_q && !is_k;
+    const bool works = inside && (is_q || a.write_kv);
+    const int d = (is_q || is_k) ? c % a.head_dim : 0;          // the first of the lane's four features within its head
+    const bool normed = (is_q || is_k) && a.eps > 0.0f, turned = (is_q || is_k) && a.rotary_dim > 0 && d < a.rotary_dim;
+    const int K = a.taps ? a.n_taps : 1;
+    const int first = t0 - (K - 1);                            // the row that staged[0 ..] holds (rows before 0 are not there)
+    if (TPW > 1 && a.taps) {      // (a wave with one token reads its few rows from memory itself: no wait for the block)
+        int n_rows = min(t0 + QKV_WIDE_TOKENS, a.n_tokens) - first;
+        for (int i = wave; i < n_rows; i += 4) {
+            int r = first + i;
+            if (r >= 0 && works) staged[i * 64 + lane] = *(const float4*)(sums + (size_t)r * a.in_stride + c);
+        }
+        __syncthreads();
+    }
+    // what does not depend on the token
+    float nwv[4] = {1.0f, 1.0f, 1.0f, 1.0f};
+    const float* nw = is_q ? a.q_weight : a.k_weight;
+    if (works && normed && nw) load4(nw + d, nwv);
+    float f0 = 0.0f, f1 = 0.0f;
+    if (works && turned) {
+        f0 = inv_freq[d >> 1];
+        f1 = d + 2 < a.rotary_dim ? inv_freq[(d >> 1) + 1] : 0.0f;
+    }
+    float tw[4][4] = {};                                       // the taps of the lane's four columns, where there are at most four
+    const float* w = a.taps ? a.taps + (size_t)c * K : nullptr;      // column c + f's taps at w[f * K ..]
+    if (works && a.taps && K <= 4) {
+#pragma unroll
+        for (int f = 0; f < 4; ++f)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (j < K) tw[f][j] = w[f * K + j];
+    }
+    float bv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (works && !a.taps && bias) load4(bias + c, bv);
+
+    for (int tt = 0; tt < QKV_WIDE_TOKENS / 4; ++tt) {
+        const int t = t0 + wave * (QKV_WIDE_TOKENS / 4) + tt;
+        if (t >= a.n_tokens) break;                            // (the whole wave: t is the wave's)
+        float x[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        const float pos = (works && turned) ? (float)positions[t] : 0.0f;
+        const int slot = (works && !is_q) ? slot_map[t] : -1;
+        if (works) {
+            if (a.taps) {
+                int e = a.token_entry[t];
+                int place = t - a.q_starts[e];
+                const float* sp = K > 1 ? a.state + (size_t)a.slots[e] * a.state_stride + c : nullptr;
+                auto row = [&](int back, float (&in)[4]) {       // the row `back` tokens before this one
+                    if (place - back >= 0) {
+                        float4 v = TPW > 1 ? staged[(t - back - first) * 64 + lane]
+                                           : *(const float4*)(sums + (size_t)(t - back) * a.in_stride + c);
+                        in[0] = v.x; in[1] = v.y; in[2] = v.z; in[3] = v.w;
+                    } else {
+                        load4(sp + (size_t)(K - 1 + place - back) * a.columns, in);
+                    }
+                };
+                if (K <= 4) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        if (j < K) {
+                            float in[4];
+                            row(K - 1 - j, in);
+#pragma unroll
+                            for (int f = 0; f < 4; ++f) x[f] = fmaf(tw[f][j], in[f], x[f]);
+                        }
+                } else {
+                    for (int j = 0; j < K; ++j) {
+                        float in[4];
+                        row(K - 1 - j, in);
+#pragma unroll
+                        for (int f = 0; f < 4; ++f) x[f] = fmaf(w[f * K + j], in[f], x[f]);
+                    }
+                }
+            } else {
+                load4(sums + (size_t)t * a.in_stride + c, x);
+#pragma unroll
+                for (int f = 0; f < 4; ++f) x[f] += bv[f];
+            }
+        }
+        // every lane takes part in the sums across lanes; a head's lanes are head_dim / 4 neighbours
+        if (a.eps > 0.0f) {
+            float ss = fmaf(x[0], x[0], fmaf(x[1], x[1], fmaf(x[2], x[2], x[3] * x[3])));
+            for (int off = 1; off < a.head_dim / 4; off <<= 1) ss += __shfl_xor(ss, off, 64);
+            if (normed) {
+                float inv = 1.0f / sqrtf(ss / (float)a.head_dim + a.eps);
+#pragma unroll
+                for (int f = 0; f < 4; ++f) x[f] = x[f] * inv * nwv[f];
+            }
+        }
+        if (!works) continue;
+        if (turned) {
+            float s, co;
+            sincosf(pos * f0, &s, &co);
+            s *= a.gain;
+            co *= a.gain;
+            float u = x[0], v = x[1];
+            x[0] = fmaf(u, co, -v * s);
+            x[1] = fmaf(v, co, u * s);
+            if (d + 2 < a.rotary_dim) {
+                sincosf(pos * f1, &s, &co);
+                s *= a.gain;
+                co *= a.gain;
+                u = x[2];
+                v = x[3];
+                x[2] = fmaf(u, co, -v * s);
+                x[3] = fmaf(v, co, u * s);
+            }
+        }
+        if (is_q) {
+            qkv_store4<T>(q + (size_t)t * a.q_stride + c, x);
+            continue;
+        }
+        if (slot < 0 || slot >= a.num_pages * a.page_size) continue;  // never write outside the cache
+        int page = slot / a.page_size, off = slot % a.page_size;
+        if (is_k) {
+            int head = (c - q_cols) / a.head_dim;
+            qkv_store4<T>(k_cache + k_cache_index(page, head, off, d, a.n_kv_heads, a.page_size, a.head_dim), x);
+        } else if (is_v) {
+            int idx = c - qk_cols, head = idx / a.v_dim, dv = idx % a.v_dim;
+#pragma unroll
+            for (int f = 0; f < 4; ++f)
+                v_cache[v_cache_index(page, head, off, dv + f, a.n_kv_heads, a.page_size, a.v_dim)] = from_f32<T>(x[f]);
+        }
+    }
+}
+
 // sums: [n_tokens, in_stride] 32-bit, a token's q heads, then its k heads, then its v heads; bias: the same columns
 // (or null); q: [n_tokens, q_stride] in `dtype`; the caches in `dtype`; slot_map: [n_tokens] page * page_size + slot.
 // n_kv_heads 0: the projection has no k and v (a mixer that reads another's cache).
@@ -176,6 +334,24 @@ extern "C" int llmrs_qkv_finish(hipStream_t stream, int dtype, const float* sums
     if (n_tokens == 0) return 0;
     QkvFinishArgs a{n_tokens, n_heads, n_kv_heads, head_dim, v_dim, in_stride, q_stride, page_size, num_pages, write_kv, eps, rotary_dim,
                     gain, q_weight, k_weight, taps, n_taps, columns, state, state_stride, q_starts, slots, token_entry};
+    // four columns a lane where the heads and the rows allow it
+    auto pieces = [](const void* p) { return p == nullptr || ((uintptr_t)p & 15) == 0; };
+    bool pow2 = head_dim >= 8 && head_dim <= 256 && (head_dim & (head_dim - 1)) == 0;
+    size_t out_piece = dtype == LLMRS_F32 ? 15 : 7;
+    bool wide = pow2 && v_dim % 4 == 0 && in_stride % 4 == 0 && q_stride % 4 == 0 && rotary_dim % 2 == 0 && pieces(sums) && pieces(bias) &&
+                pieces(q_weight) && pieces(k_weight) && ((uintptr_t)q & out_piece) == 0 && (!write_kv || ((uintptr_t)k_cache & out_piece) == 0) &&
+                (n_taps <= 1 || taps == nullptr || (pieces(state) && state_stride % 4 == 0)) && (taps == nullptr || n_taps <= 33) && (dtype == LLMRS_F32 || dtype == LLMRS_BF16);
+    if (wide) {
+        const int tpw = n_tokens > 256 ? 4 : 1;
+        dim3 wgrid(ceil_div(n_tokens, 4 * tpw), ceil_div(columns, 256));
+        size_t lds = (taps && tpw > 1) ? (size_t)(4 * tpw + n_taps - 1) * 64 * sizeof(float4) : 0;
+#define QKV_WIDE(T, TPW) qkv_finish_wide_kernel<T, TPW><<<wgrid, 256, lds, stream>>>(sums, bias, (T*)q, slot_map, (T*)k_cache, (T*)v_cache, positions, inv_freq, a)
+        if (dtype == LLMRS_F32) { if (tpw == 4) QKV_WIDE(float, 4); else QKV_WIDE(float, 1); }
+        else { if (tpw == 4) QKV_WIDE(bf16, 4); else QKV_WIDE(bf16, 1); }
+#undef QKV_WIDE
+        LLMRS_LAUNCH_CHECK("qkv_finish");
+        return 0;
+    }
     dim3 grid(ceil_div(n_tokens, 4), n_heads + 2 * n_kv_heads);
     int widest = head_dim > v_dim ? head_dim : v_dim;
     if (dtype != LLMRS_F32 && dtype != LLMRS_BF16) return llmrs_fail("qkv_finish: unknown dtype %d", dtype);

@@ -144,13 +144,16 @@ def test_the_small_kernels_around_the_two_attentions(dtype):
         k.conv_state_update(sums.cuda(), got, q_starts.cuda(), sl.cuda(), C, taps)
         assert torch.equal(got.cpu(), want), (taps, C)
     # q, k and v from the product's sums: convolved from the state on, normed with a weight, turned with a gain, into pages
-    for heads, kv, hd, vd, taps, rot in ((2, 1, 6, 4, 3, 4), (4, 2, 64, 64, 4, 32), (3, 3, 20, 36, 1, 20), (2, 2, 128, 32, 5, 0), (1, 1, 8, 8, 0, 8)):
+    # (rows of whole 16-byte pieces under heads of a power of two go to the kernel with four columns a lane, others not)
+    for heads, kv, hd, vd, taps, rot, pad in ((2, 1, 6, 4, 3, 4, 5), (4, 2, 64, 64, 4, 32, 5), (4, 2, 64, 64, 4, 32, 8), (3, 3, 20, 36, 1, 20, 0),
+                                              (2, 2, 128, 32, 5, 0, 0), (1, 1, 8, 8, 0, 8, 4), (2, 1, 16, 8, 2, 10, 0), (3, 1, 8, 12, 3, 6, 0),
+                                              (5, 5, 32, 4, 1, 32, 0), (2, 1, 256, 64, 4, 64, 0), (1, 1, 8, 8, 4, 2, 3)):
         lengths, slots, page_size, pages = [1, 6, 2, 9], [2, 0, 3, 1], 4, 8
         starts = [0]
         for n in lengths:
             starts.append(starts[-1] + n)
         T, C = starts[-1], (heads + kv) * hd + kv * vd
-        sums = torch.randn(T, C + 5, generator=g)[:, :C]
+        full = torch.randn(T, C + pad, generator=g)            # (the rows lie inside wider rows)
         tp = torch.randn(C, taps, generator=g) if taps else None
         state = torch.randn(4, max(taps - 1, 1) * C, generator=g) if taps else None
         token_entry = torch.tensor([e for e, n in enumerate(lengths) for _ in range(n)], dtype=torch.int32)
@@ -164,7 +167,7 @@ def test_the_small_kernels_around_the_two_attentions(dtype):
             q = to(torch.empty(T, heads * hd, dtype=dtype))
             kc, vc = to(torch.zeros(pages * kv * page_size * hd, dtype=dtype)), to(torch.zeros(pages * kv * page_size * vd, dtype=dtype))
             conv = None if not taps else (to(tp), to(state) if taps > 1 else None, to(q_starts), to(sl), to(token_entry))
-            kk.qkv_finish(to(sums), None, q, to(slot_map), kc, vc, heads, kv, hd, vd, page_size, pages, True, 1e-5, to(positions), to(inv_freq), rot,
+            kk.qkv_finish(to(full)[:, :C], None, q, to(slot_map), kc, vc, heads, kv, hd, vd, page_size, pages, True, 1e-5, to(positions), to(inv_freq), rot,
                           q_weight=to(qw), k_weight=to(kw), gain=1.3, conv=conv)
             outs.append((q, kc, vc))
         for want, got, what in zip(outs[0], outs[1], ("q", "keys", "values")):
