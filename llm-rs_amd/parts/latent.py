@@ -37,6 +37,8 @@ class LatentAttention(KeyedBySplitChunk, Mixer):
         self.gate = p.get("gate")
         if self.gate not in (None, "head"):
             raise ValueError(f"unknown output gate {self.gate!r} (known: head)")
+        if self.rank > 512:         # the attention kernels' widest head, which the latent vector is here
+            raise ValueError(f"a latent vector of {self.rank} numbers exceeds the 512 that the attention kernels take")
         self.recording_signature = ("attention", 1, self.rank, 0)
         leaves = {"q": "q", "dkv": "dkv", "dkv_norm": "dkv.norm", "uk": "uk", "uv": "uv", "sink": "sink", "gate": "g", "o": "o",
                   **(p.get("names") or {})}
