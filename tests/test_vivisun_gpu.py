@@ -19,7 +19,6 @@ from vivisun_cases import (BENT, CONFIGS, PAGE_SIZE, allowed_error, attention, c
 
 pytestmark = pytest.mark.gpu
 DTYPES = ["float32", "bfloat16"]
-TORCH = {"float32": torch.float32, "bfloat16": torch.bfloat16}
 
 
 def replay(engine, steps):
@@ -82,7 +81,6 @@ def test_every_head_by_its_own_matrix(heads, n_in, n_out, dtype):
     g = torch.Generator().manual_seed(heads * 1000 + n_in)
     k = kernels()
     w = (torch.randn(heads, n_out, n_in, generator=g) * n_in ** -0.5).to(dtype)
-    results = {}
     for T in (1, 8, 16, 17, 100, 600):        # (few rows, rows in one block, many: three tilings with the same sums)
         a = torch.randn(600, heads * n_in, generator=g)[:T].to(dtype)
         gate = torch.randn(T, heads, generator=g) * 2
@@ -92,7 +90,6 @@ def test_every_head_by_its_own_matrix(heads, n_in, n_out, dtype):
             k.head_product(a.cuda(), w.cuda(), got, gate=None if gt is None else gt.cuda())
             ref = want if gt is None else want * (1.0 / (1.0 + torch.exp(-gt.double())))[:, :, None]
             close(got, ref.reshape(T, heads * n_out), dtype, f"{T} rows")
-        results[T] = got.cpu()
     # rows inside wider rows (a stride), and a row's result is the same bits whatever else is in the step
     a = torch.randn(600, heads * n_in, generator=g).to(dtype)
     full = torch.empty(600, heads * n_out, dtype=dtype, device="cuda")
