@@ -8,6 +8,7 @@ import os
 from typing import Any, Callable, Dict
 
 from .llama import ConfigError, LlamaConfig
+from .gokosun import GokosunConfig
 from .lilatar import LilatarConfig
 from .tuvodra import TuvodraConfig
 from .vivisun import VivisunConfig
@@ -62,3 +63,4 @@ register_architecture("LlamaForCausalLM", LlamaConfig.from_dict)
 register_architecture("Tuvodra", TuvodraConfig.from_dict)
 register_architecture("Lilatar", LilatarConfig.from_dict)
 register_architecture("Vivisun", VivisunConfig.from_dict)
+register_architecture("Gokosun", GokosunConfig.from_dict)

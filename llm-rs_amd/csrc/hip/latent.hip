@@ -2,8 +2,11 @@
 // c is cached.  Attention then runs in the latent space (attention*.hip, one key head of width `rank` whose values are
 // its keys), between two products that carry every head's query into that space and its result out of it.
 //
-//   latent_finish: the input product's 32-bit sums -> q in the activation type; c = rmsnorm(sums_c) * weight into its
-//                  page twice: as a row of the keys [page][slot][rank], as a column of the values [page][rank][slot]
+//   latent_finish: the input product's 32-bit sums -> q in the activation type (as it is, or RMS-normed with a weight
+//                  where the queries pass a latent vector of their own); c = rmsnorm(sums_c) * weight into its page
+//                  twice: as a row of the keys [page][slot][width], as a column of the values [page][width][slot];
+//                  behind c, where the design has one, a key part rotated by position that all heads share
+//                  (width = rank + its columns)
 //   head_product:  out[t, h, :] = W[h] a[t, h, :], every head by its own small matrix, optionally times
 //                  sigmoid(gate[t, h]) computed on the 32-bit sums
 #include "cache_layout.h"
@@ -14,13 +17,49 @@ template <class T>
 __global__ __launch_bounds__(256) void latent_finish_kernel(const float* __restrict__ sums, int ld, T* __restrict__ q, int ldq,
                                                             int q_size, int rank, const float* __restrict__ weight, float eps,
                                                             const int* __restrict__ slot_map, T* __restrict__ k_cache,
-                                                            T* __restrict__ v_cache, int page_size, int num_pages, int write) {
+                                                            T* __restrict__ v_cache, int page_size, int num_pages, int write,
+                                                            const float* __restrict__ q_weight, int rot,
+                                                            const int* __restrict__ positions, const float* __restrict__ inv_freq,
+                                                            float gain) {
+    __shared__ float partial[4];
     int t = blockIdx.x;
     const float* src = sums + (size_t)t * ld;
-    for (int d = threadIdx.x; d < q_size; d += 256) q[(size_t)t * ldq + d] = from_f32<T>(src[d]);
-    if (threadIdx.x >= 64 || !write) return;
-    int lane = threadIdx.x;
+    float q_inv = 1.0f;
+    if (q_weight) {                 // the q part is a latent vector of its own: normed over its whole width
+        float ss = 0.0f;
+        for (int d = threadIdx.x; d < q_size; d += 256) ss = fmaf(src[d], src[d], ss);
+        ss = wave_sum(ss);
+        if ((threadIdx.x & 63) == 0) partial[threadIdx.x >> 6] = ss;
+        __syncthreads();
+        q_inv = 1.0f / sqrtf((partial[0] + partial[1] + partial[2] + partial[3]) / (float)q_size + eps);
+    }
+    for (int d = threadIdx.x; d < q_size; d += 256) q[(size_t)t * ldq + d] = from_f32<T>(q_weight ? src[d] * q_inv * q_weight[d] : src[d]);
+    if (threadIdx.x >= 128 || !write) return;
+    int slot = slot_map[t];
+    if (slot < 0 || slot >= num_pages * page_size) return;  // never write outside the cache
+    int page = slot / page_size, off = slot % page_size;
+    const int lane = threadIdx.x & 63, width = rank + rot;
     float x[8];            // features lane, lane + 64, ... (up to 512)
+    if (threadIdx.x >= 64) {        // the second wave: the rotated part behind c, pairs (2i, 2i + 1) by position * inv_freq[i]
+        if (rot == 0) return;
+        const float pos = (float)positions[t];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            int d = lane + 64 * i;
+            x[i] = d < rot ? src[q_size + rank + d] : 0.0f;
+            float other = __shfl_xor(x[i], 1, 64);
+            if (d < rot) {
+                float sn, cs;
+                sincosf(pos * inv_freq[d >> 1], &sn, &cs);
+                sn *= gain;
+                cs *= gain;
+                T y = from_f32<T>((d & 1) ? fmaf(x[i], cs, other * sn) : fmaf(x[i], cs, -other * sn));
+                k_cache[k_cache_index(page, 0, off, rank + d, 1, page_size, width)] = y;
+                v_cache[v_cache_index(page, 0, off, rank + d, 1, page_size, width)] = y;
+            }
+        }
+        return;
+    }
     float ss = 0.0f;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
@@ -29,35 +68,38 @@ __global__ __launch_bounds__(256) void latent_finish_kernel(const float* __restr
         ss = fmaf(x[i], x[i], ss);
     }
     float inv = 1.0f / sqrtf(wave_sum(ss) / (float)rank + eps);
-    int slot = slot_map[t];
-    if (slot < 0 || slot >= num_pages * page_size) return;  // never write outside the cache
-    int page = slot / page_size, off = slot % page_size;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
         int d = lane + 64 * i;
         if (d >= rank) continue;
         T c = from_f32<T>(x[i] * inv * weight[d]);
-        k_cache[k_cache_index(page, 0, off, d, 1, page_size, rank)] = c;
-        v_cache[v_cache_index(page, 0, off, d, 1, page_size, rank)] = c;
+        k_cache[k_cache_index(page, 0, off, d, 1, page_size, width)] = c;
+        v_cache[v_cache_index(page, 0, off, d, 1, page_size, width)] = c;
     }
 }
 
-// sums: [n_tokens, ld] 32-bit, a token's q (q_size columns), then its c (rank columns); q: [n_tokens, ldq] in `dtype`;
-// weight: [rank] 32-bit; the caches in `dtype`; slot_map: [n_tokens] page * page_size + slot.
+// sums: [n_tokens, ld] 32-bit, a token's q part (q_size columns), then its c (rank columns), then `rot` columns of a
+// key part that is rotated by position and shared by all heads; q: [n_tokens, ldq] in `dtype`: the q part as it is, or
+// (q_weight [q_size] given) RMS-normed over its width and multiplied by q_weight; weight: [rank] 32-bit; the caches in
+// `dtype`, one key head of width rank + rot: c, then the rotated part; slot_map: [n_tokens] page * page_size + slot.
 extern "C" int llmrs_latent_finish(hipStream_t stream, int dtype, const float* sums, int ld, void* q, int ldq, int n_tokens,
                                    int q_size, int rank, const float* weight, float eps, const int* slot_map, void* k_cache,
-                                   void* v_cache, int page_size, int num_pages, int write) {
-    LLMRS_REQUIRE(n_tokens >= 0 && q_size > 0 && rank > 0 && ld >= q_size + rank && ldq >= q_size, "latent_finish: bad sizes");
-    LLMRS_REQUIRE(rank <= 512, "latent_finish: a latent vector of %d numbers exceeds 512", rank);
+                                   void* v_cache, int page_size, int num_pages, int write, const float* q_weight, int rot,
+                                   const int* positions, const float* inv_freq, float gain) {
+    LLMRS_REQUIRE(n_tokens >= 0 && q_size > 0 && rank > 0 && rot >= 0 && ld >= q_size + rank + rot && ldq >= q_size, "latent_finish: bad sizes");
+    LLMRS_REQUIRE(rank <= 512 && rot <= 512, "latent_finish: a latent vector of %d numbers or a rotated part of %d exceeds 512", rank, rot);
     LLMRS_REQUIRE(eps > 0.0f && weight, "latent_finish: the norm needs its weight and a positive eps");
+    LLMRS_REQUIRE(rot == 0 || (rot % 2 == 0 && positions && inv_freq), "latent_finish: a rotated part has an even width, positions and frequencies");
     LLMRS_REQUIRE(!write || (page_size > 0 && num_pages > 0 && slot_map && k_cache && v_cache), "latent_finish: no cache to write");
     if (n_tokens == 0) return 0;
     if (dtype == LLMRS_F32)
         latent_finish_kernel<float><<<n_tokens, 256, 0, stream>>>(sums, ld, (float*)q, ldq, q_size, rank, weight, eps, slot_map,
-                                                                   (float*)k_cache, (float*)v_cache, page_size, num_pages, write);
+                                                                   (float*)k_cache, (float*)v_cache, page_size, num_pages, write,
+                                                                   q_weight, rot, positions, inv_freq, gain);
     else if (dtype == LLMRS_BF16)
         latent_finish_kernel<bf16><<<n_tokens, 256, 0, stream>>>(sums, ld, (bf16*)q, ldq, q_size, rank, weight, eps, slot_map,
-                                                                  (bf16*)k_cache, (bf16*)v_cache, page_size, num_pages, write);
+                                                                  (bf16*)k_cache, (bf16*)v_cache, page_size, num_pages, write,
+                                                                  q_weight, rot, positions, inv_freq, gain);
     else
         return llmrs_fail("latent_finish: unknown dtype %d", dtype);
     LLMRS_LAUNCH_CHECK("latent_finish");

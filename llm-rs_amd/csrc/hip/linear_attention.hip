@@ -1,6 +1,8 @@
 // Mixers whose memory is a matrix per head, S [key channel][value channel], carried from token to token in 32-bit:
 //
-//   S <- decay * S                      decay: one number per head, or one per (token, head, key channel)
+//   S <- decay * S                      decay: one number per head, or one per (token, head, key channel), or one per
+//                                       (token, head) together with a strength per (token, head) that the write is
+//                                       multiplied by: gates that move with the token
 //   u  = beta (v - S^T k)               with a write strength beta per (token, head): the delta rule;
 //   u  = v                              without: plain linear attention
 //   S <- S + k u^T;    o = S^T q        (the read-out sees the current token's write)
@@ -22,6 +24,10 @@ struct LinearScanArgs {
     const float* g; int ldg;            // [T, heads * dk] decay per key channel, or null
     const float* decay;                 // [heads] decay per head, or null (both null: none)
     const float* beta; int ldb;         // [T, heads] write strength of the delta rule, or null: plain linear attention
+    const float* tdecay;                // [T, heads] decay per (token, head) and
+    const float* ttake; int ldt;        // [T, heads] what the token's write is multiplied by, or both null
+    int v_cols;                         // columns that v holds per head; the state's columns past them (dv > v_cols) are
+                                        // written with the value 1: S's extra column is then the sum of the keys themselves
     float* state; long state_stride;    // [slots][heads][dv][dk]: a column's rows side by side, as a lane reads and leaves them
     int state_vec;                      // rows of the state may be read four at a time (dk % 4 == 0, 16-byte aligned slots)
     float* out; int ldo;                // [T, heads * dv]
@@ -57,7 +63,7 @@ __device__ __forceinline__ float column_sum(float x) {
 // A token's operands are the same for all of them: the block brings the q, k (and decay) rows of the next CHUNK tokens
 // into LDS, through registers, while it folds the current CHUNK in, so that the walk from token to token waits for LDS
 // and arithmetic only, never for memory.
-template <int P, int R, bool DELTA, bool CHANNEL_DECAY>
+template <int P, int R, bool DELTA, bool CHANNEL_DECAY, bool TOKEN_GATES = false>
 __global__ __launch_bounds__(SCAN_THREADS) void linear_scan_kernel(const int* __restrict__ q_starts, const int* __restrict__ slots,
                                                                     LinearScanArgs a) {
     constexpr int DKP = P * R;                              // rows with the idle ones
@@ -70,6 +76,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void linear_scan_kernel(const int* __
     __shared__ __attribute__((aligned(16))) float sg[CHANNEL_DECAY ? 2 : 1][CHANNEL_DECAY ? CHUNK : 1][CHANNEL_DECAY ? DKP : 4];
     __shared__ float sv[2][CHUNK][CPB];
     __shared__ float sb[2][CHUNK];
+    __shared__ float sd[TOKEN_GATES ? 2 : 1][CHUNK], st[TOKEN_GATES ? 2 : 1][CHUNK];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int part = lane & (P - 1);
     const int cb = wave * CPW + lane / P;                   // this lane's column within the block
@@ -97,7 +104,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void linear_scan_kernel(const int* __
 
     // what this thread brings of a chunk: elements tid, tid + 256, ... of [CHUNK][DKP], and one value or write strength
     constexpr int NV = (CHUNK * CPB + SCAN_THREADS - 1) / SCAN_THREADS;     // values of a chunk that a thread brings
-    float rk[NROW], rq[NROW], rg[CHANNEL_DECAY ? NROW : 1], rv[NV], rb = 1.0f;
+    float rk[NROW], rq[NROW], rg[CHANNEL_DECAY ? NROW : 1], rv[NV], rb = 1.0f, rd = 1.0f, rt = 0.0f;
     auto fetch = [&](int tc) {
 #pragma unroll
         for (int n = 0; n < NROW; ++n) {
@@ -111,9 +118,14 @@ __global__ __launch_bounds__(SCAN_THREADS) void linear_scan_kernel(const int* __
 #pragma unroll
         for (int n = 0; n < NV; ++n) {
             int idx = tid + n * SCAN_THREADS, i = idx / CPB, c = idx - i * CPB, t = tc + i, cc = blockIdx.x * CPB + c;
-            rv[n] = (idx < CHUNK * CPB && t < t1 && cc < a.dv) ? a.v[(size_t)t * a.ldv + (size_t)h * a.dv + cc] : 0.0f;
+            rv[n] = (idx < CHUNK * CPB && t < t1 && cc < a.dv) ? (cc < a.v_cols ? a.v[(size_t)t * a.ldv + (size_t)h * a.v_cols + cc] : 1.0f) : 0.0f;
         }
         if (DELTA && tid < CHUNK) rb = tc + tid < t1 ? a.beta[(size_t)(tc + tid) * a.ldb + h] : 0.0f;
+        if (TOKEN_GATES && tid < CHUNK) {
+            bool in = tc + tid < t1;
+            rd = in ? a.tdecay[(size_t)(tc + tid) * a.ldt + h] : 1.0f;
+            rt = in ? a.ttake[(size_t)(tc + tid) * a.ldt + h] : 0.0f;
+        }
     };
     auto stash = [&](int buf) {
 #pragma unroll
@@ -129,6 +141,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void linear_scan_kernel(const int* __
             if (idx < CHUNK * CPB) sv[buf][idx / CPB][idx % CPB] = rv[n];
         }
         if (DELTA && tid < CHUNK) sb[buf][tid] = rb;
+        if (TOKEN_GATES && tid < CHUNK) { sd[buf][tid] = rd; st[buf][tid] = rt; }
     };
     fetch(t0);
     stash(0);
@@ -153,19 +166,21 @@ __global__ __launch_bounds__(SCAN_THREADS) void linear_scan_kernel(const int* __
                 }
             }
             float u = sv[buf][i][cb];
+            const float now_decay = TOKEN_GATES ? sd[TOKEN_GATES ? buf : 0][i] : head_decay;
+            if constexpr (TOKEN_GATES) u *= st[TOKEN_GATES ? buf : 0][i];
             if constexpr (DELTA) {
                 float d0 = 0.0f, d1 = 0.0f;
 #pragma unroll
                 for (int x = 0; x < R; x += 2) {
-                    s[x] *= CHANNEL_DECAY ? gc[x] : head_decay;
-                    s[x + 1] *= CHANNEL_DECAY ? gc[x + 1] : head_decay;
+                    s[x] *= CHANNEL_DECAY ? gc[x] : now_decay;
+                    s[x + 1] *= CHANNEL_DECAY ? gc[x + 1] : now_decay;
                     d0 = fmaf(kc[x], s[x], d0);
                     d1 = fmaf(kc[x + 1], s[x + 1], d1);
                 }
                 u = sb[buf][i] * (u - column_sum<P>(d0 + d1));
             } else {
 #pragma unroll
-                for (int x = 0; x < R; ++x) s[x] *= CHANNEL_DECAY ? gc[x] : head_decay;
+                for (int x = 0; x < R; ++x) s[x] *= CHANNEL_DECAY ? gc[x] : now_decay;
             }
             float o0 = 0.0f, o1 = 0.0f;
 #pragma unroll
@@ -199,13 +214,19 @@ static bool entries_given(const int* q_starts, const int* slots, int n_entries) 
 // q, k: [T, qk_heads * dk]; v: [T, heads * dv]; g: [T, heads * dk] or null; decay: [heads] or null; beta: [T, heads] or
 // null (no delta correction); state: [slots][heads][dv][dk] at state_stride floats a slot, read at an entry's first
 // token and left at its last; out: [T, heads * dv].  All 32-bit.  Head h reads the q and k of head h / (heads / qk_heads).
+// tdecay, ttake: [T, heads] each or both null: S <- tdecay S + ttake k v^T.  v: [T, heads * v_cols]; with v_cols < dv the
+// columns past v_cols are written with 1 in v's place.
 extern "C" int llmrs_linear_scan(hipStream_t stream, const float* q, int ldq, const float* k, int ldk, const float* v, int ldv,
                                  const float* g, int ldg, const float* decay, const float* beta, int ldb, float* state,
                                  long state_stride, const int* q_starts, const int* slots, int n_entries, int n_tokens,
-                                 int heads, int qk_heads, int dk, int dv, float* out, int ldo) {
+                                 int heads, int qk_heads, int dk, int dv, float* out, int ldo, const float* tdecay, const float* ttake,
+                                 int ldt, int v_cols) {
     LLMRS_REQUIRE(heads > 0 && qk_heads > 0 && heads % qk_heads == 0 && dk > 0 && dv > 0, "linear_scan: bad sizes");
+    LLMRS_REQUIRE(v_cols > 0 && v_cols <= dv, "linear_scan: v holds 1 to dv columns a head, not %d", v_cols);
+    LLMRS_REQUIRE((tdecay == nullptr) == (ttake == nullptr) && (!tdecay || ldt >= heads), "linear_scan: gates per token come as a pair of [T, heads]");
+    LLMRS_REQUIRE(!tdecay || (!g && !decay && !beta), "linear_scan: gates per token go with no other decay and no delta correction");
     LLMRS_REQUIRE(dk <= 512, "linear_scan: %d key channels exceed 512", dk);
-    LLMRS_REQUIRE(ldq >= qk_heads * dk && ldk >= qk_heads * dk && ldv >= heads * dv && ldo >= heads * dv, "linear_scan: row stride too short");
+    LLMRS_REQUIRE(ldq >= qk_heads * dk && ldk >= qk_heads * dk && ldv >= heads * v_cols && ldo >= heads * dv, "linear_scan: row stride too short");
     LLMRS_REQUIRE(!g || ldg >= heads * dk, "linear_scan: the decays' rows are too short");
     LLMRS_REQUIRE(!(g && decay), "linear_scan: a decay per head or per channel, not both");
     LLMRS_REQUIRE(!beta || ldb >= heads, "linear_scan: the write strengths' rows are too short");
@@ -213,12 +234,13 @@ extern "C" int llmrs_linear_scan(hipStream_t stream, const float* q, int ldq, co
     LLMRS_REQUIRE(entries_given(q_starts, slots, n_entries), "linear_scan: bad entries");
     if (n_tokens == 0) return 0;
     int state_vec = dk % 4 == 0 && state_stride % 4 == 0 && ((uintptr_t)state & 15) == 0;
-    LinearScanArgs a{q, ldq, k, ldk, v, ldv, g, ldg, decay, beta, ldb, state, state_stride, state_vec, out, ldo, heads, qk_heads, dk, dv};
+    LinearScanArgs a{q, ldq, k, ldk, v, ldv, g, ldg, decay, beta, ldb, tdecay, ttake, ldt, v_cols, state, state_stride, state_vec, out, ldo, heads, qk_heads, dk, dv};
     // lanes to a column and rows to a lane by the number of key channels: eight rows a lane where that fills the lanes
-#define SCAN(PP, RR, D, C) linear_scan_kernel<PP, RR, D, C><<<dim3(ceil_div(dv, SCAN_WAVES * 64 / PP), heads, n_entries), SCAN_THREADS, 0, stream>>>(q_starts, slots, a)
-#define BY_SIZE(D, C) do { if (dk <= 32) SCAN(8, 4, D, C); else if (dk <= 64) SCAN(8, 8, D, C); else if (dk <= 128) SCAN(16, 8, D, C); \
-                           else if (dk <= 256) SCAN(32, 8, D, C); else SCAN(32, 16, D, C); } while (0)
-    if (beta && g) BY_SIZE(true, true); else if (beta) BY_SIZE(true, false); else if (g) BY_SIZE(false, true); else BY_SIZE(false, false);
+#define SCAN(PP, RR, D, C, ...) linear_scan_kernel<PP, RR, D, C, ##__VA_ARGS__><<<dim3(ceil_div(dv, SCAN_WAVES * 64 / PP), heads, n_entries), SCAN_THREADS, 0, stream>>>(q_starts, slots, a)
+#define BY_SIZE(D, C, ...) do { if (dk <= 32) SCAN(8, 4, D, C, ##__VA_ARGS__); else if (dk <= 64) SCAN(8, 8, D, C, ##__VA_ARGS__); \
+                                else if (dk <= 128) SCAN(16, 8, D, C, ##__VA_ARGS__); else if (dk <= 256) SCAN(32, 8, D, C, ##__VA_ARGS__); \
+                                else SCAN(32, 16, D, C, ##__VA_ARGS__); } while (0)
+    if (tdecay) BY_SIZE(false, false, true); else if (beta && g) BY_SIZE(true, true); else if (beta) BY_SIZE(true, false); else if (g) BY_SIZE(false, true); else BY_SIZE(false, false);
 #undef BY_SIZE
 #undef SCAN
     LLMRS_LAUNCH_CHECK("linear_scan");
@@ -289,18 +311,87 @@ extern "C" int llmrs_delta_prepare(hipStream_t stream, float* q, int ldq, float*
     return 0;
 }
 
+// ---- the gates of a matrix memory with exponential gates, kept in range by a running maximum -----------------------
+// Per (token, head), from the raw gate projections gi, gf (32-bit sums) and their biases:
+//   i = cap tanh((gi + bi) / cap)                  the input gate's logarithm, bent into (-cap, cap)
+//   f = log sigmoid(cap tanh((gf + bf) / cap))     the forget gate's logarithm
+//   m_t = max(f + m_(t-1), i)                      the running maximum, carried in the request's state (it starts at 0)
+//   decay = exp(f + m_(t-1) - m_t),  take = exp(i - m_t),  floor = exp(-m_t)
+// One wave for each (entry, head): the gates of 64 tokens at a time, a token a lane; the maximum walks over them in
+// order, one addition and one comparison a token, exactly as token-by-token steps would, so a prompt cut anywhere gives
+// the same bits.
+__device__ __forceinline__ float log_sigmoid_f32(float z) { return z >= 0.0f ? -log1pf(expf(-z)) : z - log1pf(expf(z)); }
+
+__global__ __launch_bounds__(64) void exp_gates_kernel(const float* __restrict__ gi, const float* __restrict__ gf, int ldg,
+                                                        const float* __restrict__ bi, const float* __restrict__ bf, float cap,
+                                                        float* __restrict__ m_state, long state_stride, const int* __restrict__ q_starts,
+                                                        const int* __restrict__ slots, float* __restrict__ decay,
+                                                        float* __restrict__ take, float* __restrict__ floor_, int ldo) {
+    const int h = blockIdx.x, e = blockIdx.y, lane = threadIdx.x;
+    const int t0 = q_starts[e], t1 = q_starts[e + 1];
+    if (t0 >= t1) return;
+    float* mp = m_state + (size_t)slots[e] * state_stride + h;
+    float m = *mp;
+    const float b_i = bi ? bi[h] : 0.0f, b_f = bf ? bf[h] : 0.0f, inv_cap = 1.0f / cap;
+    for (int tc = t0; tc < t1; tc += 64) {
+        const int t = tc + lane, n_here = min(64, t1 - tc);
+        const bool in = t < t1;
+        float i = 0.0f, f = 0.0f;
+        if (in) {
+            i = cap * tanhf((gi[(size_t)t * ldg + h] + b_i) * inv_cap);
+            f = log_sigmoid_f32(cap * tanhf((gf[(size_t)t * ldg + h] + b_f) * inv_cap));
+        }
+        float before = 0.0f, mine = 0.0f;
+        for (int j = 0; j < n_here; ++j) {
+            float fj = __shfl(f, j, 64), ij = __shfl(i, j, 64);
+            float m_new = fmaxf(fj + m, ij);
+            if (lane == j) { before = m; mine = m_new; }
+            m = m_new;
+        }
+        if (in) {
+            decay[(size_t)t * ldo + h] = expf(f + before - mine);
+            take[(size_t)t * ldo + h] = expf(i - mine);
+            floor_[(size_t)t * ldo + h] = expf(-mine);
+        }
+    }
+    if (lane == 0) *mp = m;
+}
+
+// gi, gf: [T, ldg] 32-bit, head h's raw gate at column h; bi, bf: [heads] or null; m_state: a request's maxima at
+// m_state + slot * state_stride + h; decay, take, floor: [T, ldo] 32-bit.
+extern "C" int llmrs_exp_gates(hipStream_t stream, const float* gi, const float* gf, int ldg, const float* bi, const float* bf, float cap,
+                               float* m_state, long state_stride, const int* q_starts, const int* slots, int n_entries, int n_tokens,
+                               int heads, float* decay, float* take, float* floor_, int ldo) {
+    LLMRS_REQUIRE(gi && gf && m_state && decay && take && floor_ && heads > 0 && ldg >= heads && ldo >= heads, "exp_gates: bad arguments");
+    LLMRS_REQUIRE(cap > 0.0f, "exp_gates: the gates' cap must be positive, got %g", cap);
+    LLMRS_REQUIRE(q_starts && slots && n_entries > 0 && n_entries <= 65535, "exp_gates: bad entries");
+    if (n_tokens == 0) return 0;
+    exp_gates_kernel<<<dim3(heads, n_entries), 64, 0, stream>>>(gi, gf, ldg, bi, bf, cap, m_state, state_stride, q_starts, slots, decay, take, floor_, ldo);
+    LLMRS_LAUNCH_CHECK("exp_gates");
+    return 0;
+}
+
 // ---- RMS norm in groups under a sigmoid gate ------------------------------------------------------------------------
-// out[t, c] = x[t, c] / sqrt(mean over c's group of x^2 + eps) * weight[c % weight_len] * sigmoid(gate[t, c]);
+// out[t, c] = y[t, c] / sqrt(mean over c's group of y^2 + eps) * weight[c % weight_len] * sigmoid(gate[t, c]);
 // groups of `group` consecutive columns; x and gate 32-bit, out in the activation type.  One block a (token, group).
+// y = x, whose groups lie `group_stride` columns apart.  With `floor` [T, groups]: a group of x has one more column, n,
+// behind its `group`, and y = x_scale x / (max(x_scale |n|, floor[t, group]) + den_add): a read-out divided by the
+// larger of its normaliser and a floor, before the norm.
 template <class T>
 __global__ __launch_bounds__(256) void gated_rmsnorm_kernel(const float* __restrict__ x, int ldx, const float* __restrict__ gate, int ldg,
                                                              const float* __restrict__ weight, int weight_len, int group, float eps,
-                                                             T* __restrict__ out, int ldo) {
+                                                             T* __restrict__ out, int ldo, int group_stride, const float* __restrict__ floor_,
+                                                             int ldf, float x_scale, float den_add) {
     __shared__ float partial[4];
     int t = blockIdx.x, c0 = blockIdx.y * group, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const float* xr = x + (size_t)t * ldx + c0;
+    const float* xr = x + (size_t)t * ldx + (size_t)blockIdx.y * group_stride;
+    float mul = 1.0f;
+    if (floor_) mul = x_scale / (fmaxf(fabsf(xr[group]) * x_scale, floor_[(size_t)t * ldf + blockIdx.y]) + den_add);
     float ss = 0.0f;
-    for (int d = threadIdx.x; d < group; d += 256) ss = fmaf(xr[d], xr[d], ss);
+    for (int d = threadIdx.x; d < group; d += 256) {
+        float y = xr[d] * mul;
+        ss = fmaf(y, y, ss);
+    }
     ss = wave_sum(ss);
     if (lane == 0) partial[wave] = ss;
     __syncthreads();
@@ -309,23 +400,26 @@ __global__ __launch_bounds__(256) void gated_rmsnorm_kernel(const float* __restr
     T* orow = out + (size_t)t * ldo + c0;
     for (int d = threadIdx.x; d < group; d += 256) {
         float sig = 1.0f / (1.0f + expf(-gr[d]));
-        orow[d] = from_f32<T>(xr[d] * inv * weight[(c0 + d) % weight_len] * sig);
+        orow[d] = from_f32<T>(xr[d] * mul * inv * weight[(c0 + d) % weight_len] * sig);
     }
 }
 
 extern "C" int llmrs_gated_rmsnorm(hipStream_t stream, int dtype, const float* x, int ldx, const float* gate, int ldg,
                                    const float* weight, int weight_len, int n_tokens, int n_groups, int group, float eps,
-                                   void* out, int ldo) {
+                                   void* out, int ldo, int group_stride, const float* floor_, int ldf, float x_scale, float den_add) {
     LLMRS_REQUIRE(x && gate && weight && out && n_groups > 0 && group > 0 && weight_len > 0, "gated_rmsnorm: bad arguments");
     long width = (long)n_groups * group;
-    LLMRS_REQUIRE(ldx >= width && ldg >= width && ldo >= width && n_groups <= 65535, "gated_rmsnorm: row stride too short");
+    LLMRS_REQUIRE(group_stride >= group + (floor_ ? 1 : 0), "gated_rmsnorm: the groups of x overlap");
+    LLMRS_REQUIRE(ldx >= (long)(n_groups - 1) * group_stride + group + (floor_ ? 1 : 0) && ldg >= width && ldo >= width && n_groups <= 65535,
+                  "gated_rmsnorm: row stride too short");
+    LLMRS_REQUIRE(!floor_ || ldf >= n_groups, "gated_rmsnorm: the floors' rows are too short");
     LLMRS_REQUIRE(weight_len == group || weight_len == width, "gated_rmsnorm: a weight per column of the row or of a group");
     if (n_tokens == 0) return 0;
     dim3 grid(n_tokens, n_groups);
     if (dtype == LLMRS_F32)
-        gated_rmsnorm_kernel<float><<<grid, 256, 0, stream>>>(x, ldx, gate, ldg, weight, weight_len, group, eps, (float*)out, ldo);
+        gated_rmsnorm_kernel<float><<<grid, 256, 0, stream>>>(x, ldx, gate, ldg, weight, weight_len, group, eps, (float*)out, ldo, group_stride, floor_, ldf, x_scale, den_add);
     else if (dtype == LLMRS_BF16)
-        gated_rmsnorm_kernel<bf16><<<grid, 256, 0, stream>>>(x, ldx, gate, ldg, weight, weight_len, group, eps, (bf16*)out, ldo);
+        gated_rmsnorm_kernel<bf16><<<grid, 256, 0, stream>>>(x, ldx, gate, ldg, weight, weight_len, group, eps, (bf16*)out, ldo, group_stride, floor_, ldf, x_scale, den_add);
     else
         return llmrs_fail("gated_rmsnorm: unknown dtype %d", dtype);
     LLMRS_LAUNCH_CHECK("gated_rmsnorm");

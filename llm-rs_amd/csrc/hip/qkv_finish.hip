@@ -364,3 +364,56 @@ extern "C" int llmrs_qkv_finish(hipStream_t stream, int dtype, const float* sums
     LLMRS_LAUNCH_CHECK("qkv_finish");
     return 0;
 }
+
+// ---- what some designs do to a q/k/v projection's 32-bit sums before the per-head stages above ----------------------
+// In place on sums [T, q | k | v], one block for each (token, part):
+//   q (and k) RMS-normed over the whole projection, all heads at once, and multiplied by a weight of that width
+//     (q_weight [q_cols], k_weight [k_cols]; null: the part stays as it is);
+//   v mixed with the values that an earlier layer made of the same token: v <- (1 - lambda) v + lambda first
+//     (first [T, v_cols] 32-bit, lambda one number on the device), or (keep given, first null) copied out for later
+//     layers to mix with.
+__global__ __launch_bounds__(256) void qkv_whole_kernel(float* __restrict__ sums, int ld, int q_cols, int k_cols, int v_cols,
+                                                        const float* __restrict__ q_weight, const float* __restrict__ k_weight, float eps,
+                                                        const float* __restrict__ first, int ld_first, const float* __restrict__ lambda,
+                                                        float* __restrict__ keep, int ld_keep) {
+    __shared__ float partial[4];
+    const int t = blockIdx.x, part = blockIdx.y;
+    if (part == 2) {
+        float* v = sums + (size_t)t * ld + q_cols + k_cols;
+        if (first) {
+            const float lam = *lambda;
+            const float* f = first + (size_t)t * ld_first;
+            for (int d = threadIdx.x; d < v_cols; d += 256) v[d] = (1.0f - lam) * v[d] + lam * f[d];
+        } else if (keep) {
+            float* o = keep + (size_t)t * ld_keep;
+            for (int d = threadIdx.x; d < v_cols; d += 256) o[d] = v[d];
+        }
+        return;
+    }
+    const float* w = part == 0 ? q_weight : k_weight;
+    if (!w) return;
+    const int n = part == 0 ? q_cols : k_cols;
+    float* x = sums + (size_t)t * ld + (part == 0 ? 0 : q_cols);
+    float ss = 0.0f;
+    for (int d = threadIdx.x; d < n; d += 256) ss = fmaf(x[d], x[d], ss);
+    ss = wave_sum(ss);
+    if ((threadIdx.x & 63) == 0) partial[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    const float inv = 1.0f / sqrtf((partial[0] + partial[1] + partial[2] + partial[3]) / (float)n + eps);
+    for (int d = threadIdx.x; d < n; d += 256) x[d] = x[d] * inv * w[d];
+}
+
+extern "C" int llmrs_qkv_whole(hipStream_t stream, float* sums, int ld, int n_tokens, int q_cols, int k_cols, int v_cols,
+                               const float* q_weight, const float* k_weight, float eps, const float* first, int ld_first,
+                               const float* lambda, float* keep, int ld_keep) {
+    LLMRS_REQUIRE(sums && n_tokens >= 0 && q_cols > 0 && k_cols >= 0 && v_cols >= 0 && ld >= q_cols + k_cols + v_cols, "qkv_whole: bad sizes");
+    LLMRS_REQUIRE((!q_weight && !k_weight) || eps > 0.0f, "qkv_whole: the norm needs a positive eps");
+    LLMRS_REQUIRE(!k_weight || k_cols > 0, "qkv_whole: a weight for keys that are not there");
+    LLMRS_REQUIRE(!first || (lambda && ld_first >= v_cols && !keep), "qkv_whole: mixing needs the first values' rows and lambda, and keeps nothing");
+    LLMRS_REQUIRE(!keep || ld_keep >= v_cols, "qkv_whole: the kept values' rows are too short");
+    if (n_tokens == 0) return 0;
+    qkv_whole_kernel<<<dim3(n_tokens, (first || keep) ? 3 : 2), 256, 0, stream>>>(sums, ld, q_cols, k_cols, v_cols, q_weight, k_weight, eps,
+                                                                                    first, ld_first, lambda, keep, ld_keep);
+    LLMRS_LAUNCH_CHECK("qkv_whole");
+    return 0;
+}

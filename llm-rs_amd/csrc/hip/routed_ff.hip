@@ -1,7 +1,10 @@
-// Feed-forwards without a gate projection, act(x Wup^T) Wdown^T, dense or as a mixture of experts.
+// Feed-forwards whose activation runs on a product's 32-bit sums, act(x Wup^T) Wdown^T without a gate projection or
+// act(x Wgate^T, x Wup^T) Wdown^T with one, dense or as a mixture of experts.
 //
 // The router: scores = softmax over all experts of the 32-bit logits; the `top` largest are chosen (of equal scores the
-// lower index first); an expert's weight is its score, as it is or divided by the chosen scores' sum.  The experts' up
+// lower index first); an expert's weight is its score, as it is or divided by the chosen scores' sum.  Or (score kind
+// 1) scores = sigmoid(logit) for each expert by itself, chosen by score + correction[e], weighed by the score without
+// it (divided by the chosen scores' sum + 1e-20 with `renormalize`), times `scale`.  The experts' up
 // matrices lie one under the other and their down matrices side by side, so that the experts of a token are a dense
 // feed-forward of experts * ff hidden units whose activations are multiplied by the expert's weight, zero for the
 // experts that were not chosen: the activation kernel below applies act and that weight in one pass.
@@ -61,46 +64,103 @@ __global__ __launch_bounds__(64) void route_topk_kernel(const float* __restrict_
     }
 }
 
+// Score kind 1.  One wave a token; the chosen experts' weights into weights [T, E], zero elsewhere.
+__global__ __launch_bounds__(64) void route_topk_sigmoid_kernel(const float* __restrict__ logits, int ld, float* __restrict__ weights, int ldw,
+                                                                 int E, int top, int renormalize, const float* __restrict__ correction,
+                                                                 float scale) {
+    int t = blockIdx.x, lane = threadIdx.x;
+    constexpr int PER = ROUTE_MAX_EXPERTS / 64;
+    float s[PER], c[PER], keep[PER];        // score, what the choice goes by (-inf: not there or taken), the weight kept
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        int e = lane + 64 * i;
+        bool in = e < E;
+        s[i] = in ? 1.0f / (1.0f + expf(-logits[(size_t)t * ld + e])) : 0.0f;
+        c[i] = in ? s[i] + (correction ? correction[e] : 0.0f) : -INFINITY;
+        keep[i] = 0.0f;
+    }
+    float chosen_sum = 0.0f;
+    for (int r = 0; r < top; ++r) {
+        float best = -INFINITY, best_s = 0.0f;
+        int at = 0x7fffffff;
+#pragma unroll
+        for (int i = 0; i < PER; ++i)
+            if (c[i] > best) { best = c[i]; best_s = s[i]; at = lane + 64 * i; }
+#pragma unroll
+        for (int d = 32; d > 0; d >>= 1) {
+            float ob = __shfl_xor(best, d, 64), os = __shfl_xor(best_s, d, 64);
+            int oa = __shfl_xor(at, d, 64);
+            if (ob > best || (ob == best && oa < at)) { best = ob; best_s = os; at = oa; }
+        }
+        if (at == 0x7fffffff) break;
+        chosen_sum += best_s;
+#pragma unroll
+        for (int i = 0; i < PER; ++i)
+            if (lane + 64 * i == at) { keep[i] = s[i]; c[i] = -INFINITY; }
+    }
+    float norm = (renormalize ? 1.0f / (chosen_sum + 1e-20f) : 1.0f) * scale;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        int e = lane + 64 * i;
+        if (e < E) weights[(size_t)t * ldw + e] = keep[i] * norm;
+    }
+}
+
+// score_kind 0: softmax over the experts (correction and scale are not used: null and 1); 1: a sigmoid for each expert,
+// chosen by score + correction [E] (null: none), weights times scale.
 extern "C" int llmrs_route_topk(hipStream_t stream, const float* logits, int ld, float* weights, int ldw, int n_tokens, int E, int top,
-                                int renormalize) {
+                                int renormalize, int score_kind, const float* correction, float scale) {
     LLMRS_REQUIRE(logits && weights && E > 0 && top > 0 && top <= E && ld >= E && ldw >= E, "route_topk: bad arguments");
     LLMRS_REQUIRE(E <= ROUTE_MAX_EXPERTS, "route_topk: %d experts exceed %d", E, ROUTE_MAX_EXPERTS);
+    LLMRS_REQUIRE(score_kind == 0 || score_kind == 1, "route_topk: unknown score kind %d (0: softmax, 1: sigmoid)", score_kind);
+    LLMRS_REQUIRE(score_kind == 1 || (correction == nullptr && scale == 1.0f), "route_topk: a correction or a scale goes with sigmoid scores");
     if (n_tokens <= 0) return 0;
-    route_topk_kernel<<<n_tokens, 64, 0, stream>>>(logits, ld, weights, ldw, E, top, renormalize);
+    if (score_kind == 1) route_topk_sigmoid_kernel<<<n_tokens, 64, 0, stream>>>(logits, ld, weights, ldw, E, top, renormalize, correction, scale);
+    else route_topk_kernel<<<n_tokens, 64, 0, stream>>>(logits, ld, weights, ldw, E, top, renormalize);
     LLMRS_LAUNCH_CHECK("route_topk");
     return 0;
 }
 
-// out[t, c] = act(up[t, c]) * (weights ? weights[t, c / ff] : 1), act = relu(x)^2 (kind 0); up 32-bit sums, out in the
-// activation type (one rounding).
-template <class T>
+// out[t, c] = act * (weights ? weights[t, c / ff] : 1); up 32-bit sums, out in the activation type (one rounding).
+// kind 0: act = relu(up[t, c])^2.  kind 1, a gated activation on sums whose columns are (gate_0, up_0, gate_1, up_1, ...):
+// g = min(up[t, 2c], limit), u = clamp(up[t, 2c + 1], -limit, limit), act = g * sigmoid(alpha * g) * (u + 1).
+template <class T, int KIND>
 __global__ void act_weight_kernel(const float* __restrict__ up, int ldu, const float* __restrict__ weights, int ldw, int ff, int n,
-                                  long total, T* __restrict__ out, int ldo) {
+                                  long total, T* __restrict__ out, int ldo, float limit, float alpha) {
     long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= total) return;
     long t = i / n;
     int c = (int)(i - t * n);
-    float x = fmaxf(up[(size_t)t * ldu + c], 0.0f);
-    float y = x * x;
+    float y;
+    if constexpr (KIND == 0) {
+        float x = fmaxf(up[(size_t)t * ldu + c], 0.0f);
+        y = x * x;
+    } else {
+        float2 gu = *(const float2*)(up + (size_t)t * ldu + 2 * c);
+        float g = fminf(gu.x, limit), u = fminf(fmaxf(gu.y, -limit), limit);
+        y = g / (1.0f + expf(-alpha * g)) * (u + 1.0f);
+    }
     if (weights) y *= weights[(size_t)t * ldw + c / ff];
     out[(size_t)t * ldo + c] = from_f32<T>(y);
 }
 
+// n: columns of out; up has n columns (kind 0) or 2 n (kind 1, then ldu even and up 8-byte aligned).
 extern "C" int llmrs_act_weight(hipStream_t stream, int dtype, const float* up, int ldu, const float* weights, int ldw, int ff,
-                                int n_tokens, int n, int kind, void* out, int ldo) {
-    LLMRS_REQUIRE(up && out && n > 0 && ldu >= n && ldo >= n && ff > 0 && n % ff == 0, "act_weight: bad arguments");
-    LLMRS_REQUIRE(kind == 0, "act_weight: unknown activation %d (0: squared relu)", kind);
+                                int n_tokens, int n, int kind, void* out, int ldo, float limit, float alpha) {
+    LLMRS_REQUIRE(up && out && n > 0 && ldo >= n && ff > 0 && n % ff == 0, "act_weight: bad arguments");
+    LLMRS_REQUIRE(kind == 0 || kind == 1, "act_weight: unknown activation %d (0: squared relu, 1: clamped gated sigmoid)", kind);
+    LLMRS_REQUIRE(ldu >= (kind == 1 ? 2 * n : n), "act_weight: the sums' rows are too short");
+    LLMRS_REQUIRE(kind == 0 || (ldu % 2 == 0 && ((uintptr_t)up & 7) == 0 && limit > 0.0f), "act_weight: gate and up side by side in 8-byte pairs, and a positive limit");
     LLMRS_REQUIRE(!weights || ldw >= n / ff, "act_weight: the weights' rows are too short");
     long total = (long)n_tokens * n;
     if (total <= 0) return 0;
     LLMRS_REQUIRE(ceil_div(total, 256) <= 0x7fffffff, "act_weight: too many elements for one launch");
     int blocks = ceil_div(total, 256);
-    if (dtype == LLMRS_F32)
-        act_weight_kernel<float><<<blocks, 256, 0, stream>>>(up, ldu, weights, ldw, ff, n, total, (float*)out, ldo);
-    else if (dtype == LLMRS_BF16)
-        act_weight_kernel<bf16><<<blocks, 256, 0, stream>>>(up, ldu, weights, ldw, ff, n, total, (bf16*)out, ldo);
-    else
-        return llmrs_fail("act_weight: unknown dtype %d", dtype);
+#define ACT(TT, KK) act_weight_kernel<TT, KK><<<blocks, 256, 0, stream>>>(up, ldu, weights, ldw, ff, n, total, (TT*)out, ldo, limit, alpha)
+    if (dtype == LLMRS_F32) { if (kind == 0) ACT(float, 0); else ACT(float, 1); }
+    else if (dtype == LLMRS_BF16) { if (kind == 0) ACT(bf16, 0); else ACT(bf16, 1); }
+    else return llmrs_fail("act_weight: unknown dtype %d", dtype);
+#undef ACT
     LLMRS_LAUNCH_CHECK("act_weight");
     return 0;
 }

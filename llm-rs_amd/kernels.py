@@ -178,7 +178,10 @@ class HipKernels(Kernels):
             "llmrs_dyt": [V, I, V, V, V, V, V, V, I, I, V, V, V, V],
             "llmrs_conv_state_update": [V, V, I, V, ctypes.c_long, V, V, I, I, I],
             "llmrs_sigmoid_gate": [V, I, V, I, V, I, I, I, I],
-            "llmrs_latent_finish": [V, I, V, I, V, I, I, I, I, V, F, V, V, V, I, I, I],
+            "llmrs_latent_finish": [V, I, V, I, V, I, I, I, I, V, F, V, V, V, I, I, I, V, I, V, V, F],
+            "llmrs_layernorm": [V, I, V, V, V, V, V, I, I, F],
+            "llmrs_exp_gates": [V, V, V, I, V, V, F, V, ctypes.c_long, V, V, I, I, I, V, V, V, I],
+            "llmrs_qkv_whole": [V, V, I, I, I, I, I, V, V, F, V, I, V, V, I],
             "llmrs_head_product": [V, I, V, I, V, V, I, I, I, I, I, I, V, I],
             "llmrs_fill_normal": [V, I, V, c_size_t, ctypes.c_uint64, ctypes.c_uint64, F, F],
             "llmrs_cast": [V, V, I, V, I, c_size_t],
@@ -199,13 +202,13 @@ class HipKernels(Kernels):
             "llmrs_streams_mix": [V, V, ctypes.c_long, I, V, V, V, ctypes.c_long],
             "llmrs_streams_copy_first": [V, V, ctypes.c_long, I, ctypes.c_long],
             "llmrs_qkv_finish": [V, I, V, I, V, V, I, V, V, V, I, I, I, I, I, I, I, I, F, V, V, I, V, V, F, V, I, V, ctypes.c_long, V, V, V, I],
-            "llmrs_linear_scan": [V, V, I, V, I, V, I, V, I, V, V, I, V, ctypes.c_long, V, V, I, I, I, I, I, I, V, I],
+            "llmrs_linear_scan": [V, V, I, V, I, V, I, V, I, V, V, I, V, ctypes.c_long, V, V, I, I, I, I, I, I, V, I, V, V, I, I],
             "llmrs_silu_columns": [V, V, I, I, I, I],
             "llmrs_delta_prepare": [V, V, I, V, I, V, I, V, I, V, V, I, I, I, I, F],
-            "llmrs_gated_rmsnorm": [V, I, V, I, V, I, V, I, I, I, I, F, V, I],
+            "llmrs_gated_rmsnorm": [V, I, V, I, V, I, V, I, I, I, I, F, V, I, I, V, I, F, F],
             "llmrs_rmsnorm_sum": [V, V, V, V, V, V, V, V, I, I, F, F],
-            "llmrs_route_topk": [V, V, I, V, I, I, I, I, I],
-            "llmrs_act_weight": [V, I, V, I, V, I, I, I, I, I, V, I],
+            "llmrs_route_topk": [V, V, I, V, I, I, I, I, I, I, V, F],
+            "llmrs_act_weight": [V, I, V, I, V, I, I, I, I, I, V, I, F, F],
             "llmrs_add_bias_rows": [V, V, I, V, I, I],
             "llmrs_route_counts": [V, V, I, I, I, V],
             "llmrs_route_rows": [V, V, I, I, I, V, V, V, V],
@@ -360,6 +363,17 @@ class HipKernels(Kernels):
                   self.lib.llmrs_dyt, self._stream(), _code(out.dtype), _p(out), _p(x), _p(weight), _p(bias), _p(alpha), _p(rows),
                   n, D, _p(out2), _p(w2), _p(b2), _p(a2))
 
+    def layernorm(self, out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: float,
+                  rows: Optional[torch.Tensor] = None) -> None:
+        """out[i, :] = (x[r] - mean) / sqrt(var + eps) * weight + bias with r = rows[i] or i, var the mean of the squared
+        deviations; x, weight, bias float32."""
+        n, D = out.shape
+        assert x.dtype == weight.dtype == bias.dtype == torch.float32 and x.is_contiguous() and out.is_contiguous()
+        assert x.shape[1] == D == weight.numel() == bias.numel() and weight.is_contiguous() and bias.is_contiguous()
+        assert (rows is None and n == x.shape[0]) or (rows is not None and rows.dtype == torch.int32 and rows.shape[0] == n)
+        self._run(f"layernorm {n}x{D}", n * D * (4 + out.element_size()) + D * 8, 8 * n * D, None, self.lib.llmrs_layernorm,
+                  self._stream(), _code(out.dtype), _p(out), _p(x), _p(weight), _p(bias), _p(rows), n, D, float(eps))
+
     def conv_state_update(self, sums: torch.Tensor, state: torch.Tensor, q_starts, slots, channels: int, taps: int) -> None:
         """state [slots, >= (taps - 1) * channels] float32 becomes each request's last taps - 1 rows of (old state, this
         step's rows of sums [T, channels]): what a causal convolution over `taps` taps reads before an entry's first token."""
@@ -377,18 +391,30 @@ class HipKernels(Kernels):
                   self._stream(), _code(o.dtype), _p(o), o.stride(0), _p(gate), gate.stride(0), T, N, per)
 
     def latent_finish(self, sums: torch.Tensor, q: torch.Tensor, q_size: int, rank: int, weight: torch.Tensor, eps: float, slot_map,
-                      k_cache: torch.Tensor, v_cache: torch.Tensor, page_size: int, num_pages: int, write: bool) -> None:
-        """sums [T, q | c | ...] float32 -> q [T, q_size] in the activation type, and c = rmsnorm(sums_c) * weight into the
-        cache's pages twice, as a row of `k_cache` [page][slot][rank] and as a column of `v_cache` [page][rank][slot]."""
+                      k_cache: torch.Tensor, v_cache: torch.Tensor, page_size: int, num_pages: int, write: bool,
+                      q_weight: Optional[torch.Tensor] = None, rotated=None) -> None:
+        """sums [T, q | c | rotated part | ...] float32 -> q [T, q_size] in the activation type (as it is, or with `q_weight`
+        [q_size] RMS-normed over its width and multiplied by it), and c = rmsnorm(sums_c) * weight into the cache's pages
+        twice, as a row of `k_cache` [page][slot][width] and as a column of `v_cache` [page][width][slot].
+        rotated = (columns, positions, inv_freq [columns / 2], gain): that many columns behind c are a key part that all
+        heads share; its features (2i, 2i + 1) are turned by positions[t] * inv_freq[i], cosine and sine times gain, and
+        written behind c (width = rank + columns; else width = rank)."""
         T = sums.shape[0]
-        assert sums.dtype == weight.dtype == torch.float32 and sums.stride(1) == 1 and sums.shape[1] >= q_size + rank
+        rot, positions, inv_freq, gain = rotated if rotated is not None else (0, None, None, 1.0)
+        width = rank + rot
+        assert sums.dtype == weight.dtype == torch.float32 and sums.stride(1) == 1 and sums.shape[1] >= q_size + width
         assert q.shape == (T, q_size) and q.stride(1) == 1 and weight.numel() == rank
+        assert q_weight is None or (q_weight.dtype == torch.float32 and q_weight.numel() == q_size and q_weight.is_contiguous())
+        if rot:
+            assert rot % 2 == 0 and positions.dtype == torch.int32 and positions.shape[0] == T
+            assert inv_freq.dtype == torch.float32 and inv_freq.numel() == rot // 2 and inv_freq.is_contiguous()
         if write:
             assert k_cache.dtype == v_cache.dtype == q.dtype and k_cache.is_contiguous() and v_cache.is_contiguous()
-            assert k_cache.numel() == v_cache.numel() == num_pages * page_size * rank and slot_map.dtype == torch.int32 and slot_map.shape[0] == T
-        self._run("latent_finish", T * (q_size + rank) * (4 + q.element_size()) + T * rank * q.element_size(), 4 * T * rank, None,
+            assert k_cache.numel() == v_cache.numel() == num_pages * page_size * width and slot_map.dtype == torch.int32 and slot_map.shape[0] == T
+        self._run("latent_finish", T * (q_size + width) * (4 + q.element_size()) + T * width * q.element_size(), 4 * T * width, None,
                   self.lib.llmrs_latent_finish, self._stream(), _code(q.dtype), _p(sums), sums.stride(0), _p(q), q.stride(0), T, q_size,
-                  rank, _p(weight), float(eps), _p(slot_map), _p(k_cache), _p(v_cache), page_size, num_pages, int(write))
+                  rank, _p(weight), float(eps), _p(slot_map), _p(k_cache), _p(v_cache), page_size, num_pages, int(write),
+                  _p(q_weight), int(rot), _p(positions) if rot else None, _p(inv_freq) if rot else None, float(gain))
 
     def head_product(self, a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gate: Optional[torch.Tensor] = None) -> None:
         """Every head by its own matrix: out[t, h, :] = w[h] @ a[t, h, :] with w [heads, n_out, n_in] (each [out, in]),
@@ -636,27 +662,68 @@ class HipKernels(Kernels):
 
     def linear_scan(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, state: torch.Tensor, q_starts, slots, heads: int,
                     qk_heads: int, dk: int, dv: int, out: torch.Tensor, decay: Optional[torch.Tensor] = None,
-                    g: Optional[torch.Tensor] = None, beta: Optional[torch.Tensor] = None) -> None:
+                    g: Optional[torch.Tensor] = None, beta: Optional[torch.Tensor] = None, gates=None, v_cols: int = 0) -> None:
         """Per head a matrix S [dk, dv] carried from token to token: S <- decay S (decay [heads], or g [T, heads * dk] a
         key channel); u = beta (v - S^T k) (beta [T, heads]; None: u = v); S <- S + k u^T; out = S^T q.  q, k
         [T, qk_heads * dk], v and out [T, heads * dv], all float32 with unit column stride; state [slots, >= heads * dk * dv]
         float32, laid out [heads][dv][dk] (a value channel's key channels side by side), read at an entry's first token
-        and left at its last."""
+        and left at its last.  gates = (decay, take), [T, heads] each: S <- decay S + take k v^T, gates that move with the
+        token.  v_cols (< dv): v holds only so many columns a head, [T, heads * v_cols]; the others are written with 1 in
+        v's place, so that a column of S past v_cols is the gated sum of the keys themselves."""
         T = q.shape[0]
-        for t in (q, k, v, out, g, beta):
+        tdecay, ttake = gates if gates is not None else (None, None)
+        v_cols = int(v_cols) or dv
+        for t in (q, k, v, out, g, beta, tdecay, ttake):
             assert t is None or (t.dtype == torch.float32 and t.stride(1) == 1 and t.shape[0] == T)
-        assert q.shape[1] == k.shape[1] == qk_heads * dk and v.shape[1] == out.shape[1] == heads * dv
+        assert q.shape[1] == k.shape[1] == qk_heads * dk and v.shape[1] == heads * v_cols and out.shape[1] == heads * dv and 0 < v_cols <= dv
+        assert gates is None or (tdecay.shape[1] == ttake.shape[1] == heads and tdecay.stride(0) == ttake.stride(0)
+                                 and decay is None and g is None and beta is None)
         assert state.dtype == torch.float32 and state.stride(-1) == 1 and state.shape[1] >= heads * dk * dv
         assert q_starts.dtype == slots.dtype == torch.int32 and q_starts.numel() == slots.numel() + 1
         assert decay is None or (decay.dtype == torch.float32 and decay.numel() == heads and decay.is_contiguous())
         assert g is None or g.shape[1] == heads * dk
         assert beta is None or beta.shape[1] == heads
-        kind = ("delta" if beta is not None else "decay") + (" by channel" if g is not None else "")
+        kind = ("delta" if beta is not None else "decay") + (" by channel" if g is not None else " by token" if gates is not None else "")
         self._run(f"linear_scan {T}x{heads}x{dk}x{dv} {kind}", T * (2 * qk_heads * dk + (heads * dk if g is not None else 0) + 2 * heads * dv) * 4
                   + slots.numel() * heads * dk * dv * 8, (7 if beta is not None else 5) * T * heads * dk * dv, None,
                   self.lib.llmrs_linear_scan, self._stream(), _p(q), q.stride(0), _p(k), k.stride(0), _p(v), v.stride(0),
                   _p(g), 0 if g is None else g.stride(0), _p(decay), _p(beta), 0 if beta is None else beta.stride(0),
-                  _p(state), state.stride(0), _p(q_starts), _p(slots), slots.numel(), T, heads, qk_heads, dk, dv, _p(out), out.stride(0))
+                  _p(state), state.stride(0), _p(q_starts), _p(slots), slots.numel(), T, heads, qk_heads, dk, dv, _p(out), out.stride(0),
+                  _p(tdecay), _p(ttake), 0 if gates is None else tdecay.stride(0), v_cols)
+
+    def exp_gates(self, gi: torch.Tensor, gf: torch.Tensor, bias_i, bias_f, cap: float, m_state: torch.Tensor, q_starts, slots,
+                  decay: torch.Tensor, take: torch.Tensor, floor: torch.Tensor) -> None:
+        """The gates of a matrix memory with exponential gates, per (token, head), float32: with i = cap tanh((gi + bias_i)
+        / cap), f = log sigmoid(cap tanh((gf + bias_f) / cap)) and the running maximum m_t = max(f + m_(t-1), i) carried in
+        m_state [slots, heads] (read at an entry's first token, left at its last): decay = exp(f + m_(t-1) - m_t),
+        take = exp(i - m_t), floor = exp(-m_t).  gi, gf [T, heads] (columns of a product's sums, equal row strides)."""
+        T, H = gi.shape
+        for t in (gi, gf, decay, take, floor):
+            assert t.dtype == torch.float32 and t.stride(1) == 1 and tuple(t.shape) == (T, H)
+        assert gi.stride(0) == gf.stride(0) and decay.stride(0) == take.stride(0) == floor.stride(0)
+        for b in (bias_i, bias_f):
+            assert b is None or (b.dtype == torch.float32 and b.numel() == H and b.is_contiguous())
+        assert m_state.dtype == torch.float32 and m_state.stride(-1) == 1 and m_state.shape[1] >= H
+        assert q_starts.dtype == slots.dtype == torch.int32 and q_starts.numel() == slots.numel() + 1
+        self._run(f"exp_gates {T}x{H}", T * H * 20, 40 * T * H, None, self.lib.llmrs_exp_gates, self._stream(), _p(gi), _p(gf), gi.stride(0),
+                  _p(bias_i), _p(bias_f), float(cap), _p(m_state), m_state.stride(0), _p(q_starts), _p(slots), slots.numel(), T, H,
+                  _p(decay), _p(take), _p(floor), decay.stride(0))
+
+    def qkv_whole(self, sums: torch.Tensor, q_cols: int, k_cols: int, v_cols: int, q_weight, k_weight, eps: float,
+                  first: Optional[torch.Tensor] = None, lam: Optional[torch.Tensor] = None, keep: Optional[torch.Tensor] = None) -> None:
+        """In place on sums [T, q | k | v] float32: q (k) RMS-normed over the whole projection and multiplied by q_weight
+        [q_cols] (k_weight [k_cols]; None: left as it is); v <- (1 - lam) v + lam first with first [T, v_cols] float32 and
+        lam one number on the device, or (keep [T, v_cols] given instead) v copied out for a later layer to mix with."""
+        T = sums.shape[0]
+        assert sums.dtype == torch.float32 and sums.stride(1) == 1 and sums.shape[1] >= q_cols + k_cols + v_cols
+        for w, n in ((q_weight, q_cols), (k_weight, k_cols)):
+            assert w is None or (w.dtype == torch.float32 and w.numel() == n and w.is_contiguous())
+        for t in (first, keep):
+            assert t is None or (t.dtype == torch.float32 and t.stride(1) == 1 and tuple(t.shape) == (T, v_cols))
+        assert first is None or (lam is not None and lam.dtype == torch.float32 and lam.numel() == 1 and keep is None)
+        self._run("qkv_whole", T * (q_cols + k_cols + v_cols) * 8, 4 * T * (q_cols + k_cols + v_cols), None, self.lib.llmrs_qkv_whole,
+                  self._stream(), _p(sums), sums.stride(0), T, q_cols, k_cols, v_cols, _p(q_weight), _p(k_weight), float(eps),
+                  _p(first), 0 if first is None else first.stride(0), _p(lam), _p(keep), 0 if keep is None else keep.stride(0))
 
     def silu_columns(self, x: torch.Tensor, col0: int, n: int) -> None:
         """x[:, col0:col0 + n] <- silu of itself; x float32 with unit column stride."""
@@ -678,15 +745,21 @@ class HipKernels(Kernels):
                   self.lib.llmrs_delta_prepare, self._stream(), _p(q), q.stride(0), _p(k), k.stride(0), _p(a), a.stride(0),
                   _p(b), b.stride(0), _p(A_log), _p(dt_bias), T, heads, qk_heads, dk, float(unit_eps))
 
-    def gated_rmsnorm(self, out: torch.Tensor, x: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, group: int, eps: float) -> None:
-        """out[t, c] = x[t, c] / sqrt(mean of x^2 over c's group of `group` columns + eps) * weight[c % len(weight)] *
-        sigmoid(gate[t, c]); x, gate float32, weight float32 of a group's or a row's length."""
-        T, W = x.shape
+    def gated_rmsnorm(self, out: torch.Tensor, x: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, group: int, eps: float,
+                      floor: Optional[torch.Tensor] = None, x_scale: float = 1.0, den_add: float = 0.0) -> None:
+        """out[t, c] = y[t, c] / sqrt(mean of y^2 over c's group of `group` columns + eps) * weight[c % len(weight)] *
+        sigmoid(gate[t, c]); x, gate float32, weight float32 of a group's or a row's length.  y = x; or, with floor
+        [T, groups] float32, x has one more column n behind each group (x [T, groups * (group + 1)]) and
+        y = x_scale x / (max(x_scale |n|, floor) + den_add)."""
+        T, W = gate.shape
+        stride = group + (1 if floor is not None else 0)
         assert x.dtype == gate.dtype == weight.dtype == torch.float32 and x.stride(1) == gate.stride(1) == out.stride(1) == 1
-        assert gate.shape == x.shape and out.shape == x.shape and W % group == 0 and weight.numel() in (group, W) and weight.is_contiguous()
+        assert out.shape == gate.shape and W % group == 0 and x.shape == (T, W // group * stride) and weight.numel() in (group, W) and weight.is_contiguous()
+        assert floor is None or (floor.dtype == torch.float32 and floor.stride(1) == 1 and tuple(floor.shape) == (T, W // group))
         self._run(f"gated_rmsnorm {T}x{W}", T * W * (8 + out.element_size()), 8 * T * W, None,
                   self.lib.llmrs_gated_rmsnorm, self._stream(), _code(out.dtype), _p(x), x.stride(0), _p(gate), gate.stride(0),
-                  _p(weight), weight.numel(), T, W // group, int(group), float(eps), _p(out), out.stride(0))
+                  _p(weight), weight.numel(), T, W // group, int(group), float(eps), _p(out), out.stride(0), stride, _p(floor),
+                  0 if floor is None else floor.stride(0), float(x_scale), float(den_add))
 
     def rmsnorm_sum(self, out: torch.Tensor, inputs, coef: float, eps: float) -> None:
         """out += coef * sum of rmsnorm(x + bias) * weight over `inputs`, one or two (x [T, D], bias [D] or None,
@@ -702,13 +775,20 @@ class HipKernels(Kernels):
         self._run(f"rmsnorm_sum {T}x{D} of {len(inputs)}", T * D * 4 * (2 + len(inputs)), 6 * len(inputs) * T * D, None,
                   self.lib.llmrs_rmsnorm_sum, self._stream(), _p(out), *flat, T, D, float(coef), float(eps))
 
-    def route_topk(self, logits: torch.Tensor, weights: torch.Tensor, top: int, renormalize: bool = False) -> None:
+    def route_topk(self, logits: torch.Tensor, weights: torch.Tensor, top: int, renormalize: bool = False, score: str = "softmax",
+                   correction: Optional[torch.Tensor] = None, scale: float = 1.0) -> None:
         """weights[t, e] = softmax(logits[t])[e] for the `top` experts with the largest scores (of equal ones the lower
-        index), 0 for the others; with `renormalize` divided by the chosen scores' sum.  Both float32 [T, experts]."""
+        index), 0 for the others; with `renormalize` divided by the chosen scores' sum.  Both float32 [T, experts].
+        score = "sigmoid": an expert's score is sigmoid(logit); the choice goes by score + correction [experts] (None:
+        by the score), the weight is the score without it (with `renormalize` divided by the chosen scores' sum + 1e-20),
+        times scale."""
         assert logits.dtype == weights.dtype == torch.float32 and logits.stride(1) == weights.stride(1) == 1 and logits.shape == weights.shape
         T, E = logits.shape
+        kind = {"softmax": 0, "sigmoid": 1}[score]
+        assert correction is None or (kind == 1 and correction.dtype == torch.float32 and correction.numel() == E and correction.is_contiguous())
+        assert kind == 1 or scale == 1.0
         self._run(f"route_topk {T}x{E}", T * E * 8, 8 * T * E, None, self.lib.llmrs_route_topk, self._stream(), _p(logits),
-                  logits.stride(0), _p(weights), weights.stride(0), T, E, int(top), int(bool(renormalize)))
+                  logits.stride(0), _p(weights), weights.stride(0), T, E, int(top), int(bool(renormalize)), kind, _p(correction), float(scale))
 
     def route_counts(self, weights: torch.Tensor, counts: torch.Tensor) -> None:
         """counts[e] = how many tokens chose expert e (weights[t, e] > 0); weights float32 [T, E], counts int32 [E]."""
@@ -737,14 +817,18 @@ class HipKernels(Kernels):
         self._run(f"combine_rows {h.shape[0]}x{h.shape[1]}", (y.numel() + 2 * h.numel()) * 4, y.numel(), None, self.lib.llmrs_combine_rows,
                   self._stream(), _p(h), h.stride(0), _p(y), y.stride(0), _p(row_of), h.shape[0], row_of.shape[1], h.shape[1])
 
-    def act_weight(self, out: torch.Tensor, up: torch.Tensor, weights: Optional[torch.Tensor], ff: int) -> None:
-        """out[t, c] = relu(up[t, c])^2 * (weights[t, c // ff] if weights is given); up, weights float32."""
-        T, N = up.shape
-        assert up.dtype == torch.float32 and up.stride(1) == 1 and out.shape == up.shape and out.stride(1) == 1 and N % ff == 0
+    def act_weight(self, out: torch.Tensor, up: torch.Tensor, weights: Optional[torch.Tensor], ff: int, activation: str = "relu2",
+                   limit: float = 0.0, alpha: float = 1.0) -> None:
+        """out[t, c] = act * (weights[t, c // ff] if weights is given); up, weights float32.  "relu2": act =
+        relu(up[t, c])^2.  "clamped_glu": up holds (gate, up) side by side, [T, 2 N]; with g = min(up[t, 2c], limit) and
+        u = clamp(up[t, 2c + 1], -limit, limit), act = g sigmoid(alpha g) (u + 1)."""
+        T, N = out.shape
+        kind = {"relu2": 0, "clamped_glu": 1}[activation]
+        assert up.dtype == torch.float32 and up.stride(1) == 1 and up.shape == (T, N * (2 if kind == 1 else 1)) and out.stride(1) == 1 and N % ff == 0
         assert weights is None or (weights.dtype == torch.float32 and weights.stride(1) == 1 and tuple(weights.shape) == (T, N // ff))
-        self._run(f"act_weight {T}x{N}", T * N * (4 + out.element_size()), 3 * T * N, None,
+        self._run(f"act_weight {T}x{N}", T * N * (4 * (kind + 1) + out.element_size()), (3 + 8 * kind) * T * N, None,
                   self.lib.llmrs_act_weight, self._stream(), _code(out.dtype), _p(up), up.stride(0), _p(weights),
-                  0 if weights is None else weights.stride(0), int(ff), T, N, 0, _p(out), out.stride(0))
+                  0 if weights is None else weights.stride(0), int(ff), T, N, kind, _p(out), out.stride(0), float(limit), float(alpha))
 
     def scan_carry_floats(self, n_tokens: int, n_entries: int, longest: int, per_place: int) -> int:
         """Room (in floats) for what the chunks of a recurrence hand on, `per_place` floats for each chunk's place;

@@ -6,9 +6,9 @@ from . import attention, block, hyper, latent, linear, mlp, norm, recurrent, rop
 from .attention import Attention
 from .latent import LatentAttention
 from .block import ParallelBlock, PreNormBlock, SandwichBlock
-from .linear import DeltaRule, Lightning, Parallel
-from .mlp import PlainFF, RoutedFF, SwiGLU
+from .linear import MLSTM, DeltaRule, Lightning, Parallel
+from .mlp import ClampedGLU, PlainFF, RoutedFF, SwiGLU
 from .hyper import HyperBlock, HyperConnection
-from .norm import DynamicTanh, GroupRMSNorm, RMSNorm
+from .norm import DynamicTanh, GroupRMSNorm, LayerNorm, RMSNorm
 from .recurrent import Mamba1, MinGRU
 from .rope import RotaryEncoding, rope_inv_freq

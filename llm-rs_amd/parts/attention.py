@@ -22,7 +22,11 @@ last conv - 1 projected rows are kept in its slot beside the pages), `qk_norm_we
 weight of head_dim numbers, one tensor for q and one for k, shared by the heads), a rotation with a `gain` (cosine and
 sine both enlarged: the position encoding says so), `gate` = "feature" | "head" (the heads' outputs are multiplied by
 sigmoid(Wg x), one gate for every feature of every head or one for each head, before the output projection; the gate's
-rows ride in the q/k/v product), `names` (the leaves of the tensors' names).  With any of them the q/k/v product leaves
+rows ride in the q/k/v product), `qk_norm_scope` = "projection" (the q/k norm runs over the whole projection, all heads
+at once, with a weight of that width, instead of head by head), `value_mix` = "first" | "later" (the values of a
+"later" layer become (1 - lambda) v + lambda v_first before they are cached, v_first the values that the "first" such
+layer made of the same token in the same step and lambda the layer's one number, tensor leaf `vmix`; the "first" layer
+holds the tensor too and does not use it), `names` (the leaves of the tensors' names).  With any of them the q/k/v product leaves
 32-bit sums, and one kernel convolves, adds the biases, norms q and k, rotates them (a rotation that the kernels fuse,
 angles in 32-bit) and writes k and v into their pages.
 
@@ -121,25 +125,39 @@ class Attention(KeyedBySplitChunk, Mixer):
             raise ValueError(f"unknown output gate {self.gate!r} (known: feature, head)")
         if self.qk_norm_weight and not self.qk_norm_eps > 0:
             raise ValueError("a q/k norm with a weight needs its eps (qk_norm_eps)")
+        self.norm_whole = p.get("qk_norm_scope", "head") == "projection"
+        if p.get("qk_norm_scope", "head") not in ("head", "projection"):
+            raise ValueError(f"unknown scope of the q/k norm {p.get('qk_norm_scope')!r} (known: head, projection)")
+        if self.norm_whole and not (self.qk_norm_weight and self.kv_proj):
+            raise ValueError("a q/k norm over the whole projection has a weight, and keys of the mixer's own")
+        self.value_mix = p.get("value_mix")
+        if self.value_mix not in (None, "first", "later"):
+            raise ValueError(f"unknown part in the mix of values {self.value_mix!r} (known: first, later)")
+        if self.value_mix is not None and not self.kv_proj:
+            raise ValueError("values that are mixed are the mixer's own")
+        if (self.norm_whole or self.value_mix is not None) and (self.taps > 0 or self.has_bias):
+            raise ValueError("a q/k norm over the whole projection and a mix of values work on the projection's sums as they are: "
+                             "with neither convolutions nor biases")
         if self.taps > 0 and (not self.kv_proj or self.has_bias):
             raise ValueError("convolutions on q, k and v go with neither biases nor a cache that another mixer wrote")
         self.gate_size = {None: 0, "feature": self.o_size, "head": self.heads}[self.gate]
         self.gain = float(getattr(self.position, "gain", 1.0)) if self.position is not None else 1.0
         # q and k are prepared by a kernel of their own between the product and attention
         self.prepared = (self.has_bias or self.qk_norm_eps > 0 or self.distance is not None or self.value_dim != self.head_dim
-                         or self.softcap > 0 or self.keep_first > 0 or self.taps > 1 or self.gate is not None or self.gain != 1.0)
+                         or self.softcap > 0 or self.keep_first > 0 or self.taps > 1 or self.gate is not None or self.gain != 1.0
+                         or self.value_mix is not None)
         if self.prepared and self.position is not None and self.position.rotary() is None:
             raise ValueError("a position encoding that is no rotation together with biases, a q/k norm, a distance penalty, a soft cap, "
                              "kept first keys or values of another width is not built")
         leaves = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
                   "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias", "o_bias": "o_proj.bias", "r1": "r1", "r2": "r2",
                   "q_norm": "q_norm.weight", "k_norm": "k_norm.weight", "q_conv": "q_conv.weight", "k_conv": "k_conv.weight",
-                  "v_conv": "v_conv.weight", "gate": "gate_proj.weight", **(p.get("names") or {})}
+                  "v_conv": "v_conv.weight", "gate": "gate_proj.weight", "value_mix": "vmix", **(p.get("names") or {})}
         self.names = {key: self.name(leaf) for key, leaf in leaves.items()}
         self.w_qkv = None
         self.w_o = None
         self.bias = self.o_bias = self.r1 = self.r2 = None
-        self.q_norm = self.k_norm = self.conv = None
+        self.q_norm = self.k_norm = self.conv = self.mix = None
         # Set by a part that holds this mixer and adds the output projection's bias itself, in a pass over the output
         # that it makes anyway (it reads the bias from `o_bias`): `forward` then leaves the bias out.
         self.output_bias_left_to_holder = False
@@ -161,9 +179,11 @@ class Attention(KeyedBySplitChunk, Mixer):
             t[n["r1"]] = TensorSpec((self.heads,), "normal:0.5:0.2")
             t[n["r2"]] = TensorSpec((self.heads,), "normal:0.5:0.05")     # 1 + r2 (i - j) must stay positive
         if self.qk_norm_weight:
-            t[n["q_norm"]] = TensorSpec((self.head_dim,), "norm")
+            t[n["q_norm"]] = TensorSpec((self.q_size if self.norm_whole else self.head_dim,), "norm")
             if self.kv_proj:
-                t[n["k_norm"]] = TensorSpec((self.head_dim,), "norm")
+                t[n["k_norm"]] = TensorSpec((self.kv_size if self.norm_whole else self.head_dim,), "norm")
+        if self.value_mix is not None:
+            t[n["value_mix"]] = TensorSpec((), "normal:0.3:0.1")
         if self.taps > 0:
             t[n["q_conv"]] = TensorSpec((self.q_size, self.taps), "normal:0.0:0.4")
             t[n["k_conv"]] = TensorSpec((self.kv_size, self.taps), "normal:0.0:0.4")
@@ -196,8 +216,11 @@ class Attention(KeyedBySplitChunk, Mixer):
         self.w_qkv = torch.cat(parts, dim=0).contiguous()
         self.w_o = get("o")
         if self.qk_norm_weight:         # (a head's features are listed in the order its rotation pairs them in)
-            self.q_norm = self._pair_neighbours(get32("q_norm").unsqueeze(1), 1).squeeze(1).contiguous()
-            self.k_norm = self._pair_neighbours(get32("k_norm").unsqueeze(1), 1).squeeze(1).contiguous() if self.kv_proj else None
+            hq, hk = (self.heads, self.kv_heads) if self.norm_whole else (1, 1)
+            self.q_norm = self._pair_neighbours(get32("q_norm").unsqueeze(1), hq).squeeze(1).contiguous()
+            self.k_norm = self._pair_neighbours(get32("k_norm").unsqueeze(1), hk).squeeze(1).contiguous() if self.kv_proj else None
+        if self.value_mix is not None:
+            self.mix = get32("value_mix").reshape(1)        # stays on the device: the kernel reads it there
         if self.taps > 0:               # the taps of q | k | v one under the other, as the product's columns are
             self.conv = torch.cat([self._pair_neighbours(get32("q_conv"), self.heads), self._pair_neighbours(get32("k_conv"), self.kv_heads),
                                    get32("v_conv")], dim=0).contiguous()
@@ -219,9 +242,12 @@ class Attention(KeyedBySplitChunk, Mixer):
         if self.gate is not None:
             out[n["gate"]] = w[self.qkv_width:].contiguous()
         if self.qk_norm_weight:
-            out[n["q_norm"]] = self._pair_neighbours(self.q_norm.cpu().unsqueeze(1), 1, undo=True).squeeze(1).contiguous()
+            hq, hk = (self.heads, self.kv_heads) if self.norm_whole else (1, 1)
+            out[n["q_norm"]] = self._pair_neighbours(self.q_norm.cpu().unsqueeze(1), hq, undo=True).squeeze(1).contiguous()
             if self.kv_proj:
-                out[n["k_norm"]] = self._pair_neighbours(self.k_norm.cpu().unsqueeze(1), 1, undo=True).squeeze(1).contiguous()
+                out[n["k_norm"]] = self._pair_neighbours(self.k_norm.cpu().unsqueeze(1), hk, undo=True).squeeze(1).contiguous()
+        if self.value_mix is not None:
+            out[n["value_mix"]] = self.mix.cpu().reshape(())
         if self.taps > 0:
             c = self.conv.cpu()
             out[n["q_conv"]] = self._pair_neighbours(c[:self.q_size], self.heads, undo=True).contiguous()
@@ -269,14 +295,24 @@ class Attention(KeyedBySplitChunk, Mixer):
         C = self.qkv_columns
         sums = ctx.workspace("attn.sums", (T, self.w_qkv.shape[0]), torch.float32)
         k.gemm(x, self.w_qkv, sums, EPI_STORE_F32, ctx.gemm_workspace(x, self.w_qkv))
+        eps, q_weight, k_weight = self.qk_norm_eps, self.q_norm, self.k_norm
+        if self.norm_whole or self.value_mix is not None:
+            # the norms over the whole projection and the mix of the values, in place on the sums; the first mixing
+            # layer's values stay in a buffer of their own for the later ones of the step
+            first = ctx.workspace("attn.value_first", (T, self.v_size), torch.float32) if self.value_mix is not None else None
+            k.qkv_whole(sums, self.q_size, self.kv_size, self.v_size, q_weight if self.norm_whole else None,
+                        k_weight if self.norm_whole else None, eps, first=first if self.value_mix == "later" else None,
+                        lam=self.mix if self.value_mix == "later" else None, keep=first if self.value_mix == "first" else None)
+            if self.norm_whole:
+                eps, q_weight, k_weight = 0.0, None, None
         q = ctx.workspace("attn.qkv", (T, self.q_size), self.dtype)
         rotary = self.position.rotary() if self.position is not None else None
         inv_freq, rotary_dim = (None, 0) if rotary is None else rotary[:2]
         # (one tap: every channel times its number, and nothing to remember)
         conv = (self.conv, conv_state, ctx.q_starts, ctx.slots, ctx.token_entry) if self.taps > 0 else None
         k.qkv_finish(sums[:, :C], self.bias, q, ctx.slot_maps[g], cache.k, cache.v, self.heads, n_kv, self.head_dim, self.value_dim,
-                     cache.page_size, cache.num_pages, write, self.qk_norm_eps, ctx.positions, inv_freq, rotary_dim,
-                     q_weight=self.q_norm, k_weight=self.k_norm, gain=self.gain, conv=conv)
+                     cache.page_size, cache.num_pages, write, eps, ctx.positions, inv_freq, rotary_dim,
+                     q_weight=q_weight, k_weight=k_weight, gain=self.gain, conv=conv)
         if self.taps > 1:
             k.conv_state_update(sums[:, :C], conv_state, ctx.q_starts, ctx.slots, C, self.taps)
         o = ctx.workspace("attn.out", (T, self.o_size), self.dtype)

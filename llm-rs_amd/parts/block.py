@@ -3,7 +3,8 @@
 halves, norms after the parts) is another subclass of `Block`, registered under
 its own name; the parts it needs beyond these four come under the names the
 layer's spec gives them in `extra`.  "sandwich": a norm before and after each half.
-"parallel": both halves read the stream as it was, each through a norm of its own."""
+"parallel": both halves read the stream as it was, each through a norm of its own or both through the one norm the
+layer has."""
 from __future__ import annotations
 
 import torch
@@ -72,25 +73,22 @@ register_block("sandwich", SandwichBlock)
 
 
 class ParallelBlock(Block):
-    """Both halves read the same stream, each through its own norm, and both add into it:
-    h <- h + mixer(mixer_norm(h)) + feed_forward(feed_forward_norm(h)).  The two norms run before either half touches
-    the stream (in one launch where the norms can: `forward_with`); the sums are 32-bit.  A layer may have no
-    feed-forward."""
+    """Both halves read the same stream and both add into it: h <- h + mixer(mixer_norm(h)) + feed_forward(n(h)), where
+    n is the feed-forward's own norm or, for a layer that has one norm only, the mixer's: then both halves read the same
+    normed rows.  The norms run before either half touches the stream (two in one launch where the norms can:
+    `forward_with`); the sums are 32-bit.  A layer may have no feed-forward."""
     needs = ("mixer", "mixer_norm")
-
-    def __init__(self, named):
-        super().__init__(named)
-        if self.feed_forward is not None and self.feed_forward_norm is None:
-            raise ValueError("block arrangement ParallelBlock needs the parts feed_forward_norm")
 
     def forward(self, ctx, h, cache):
         T, D = h.shape
         ctx.note_left(h, None)
         ctx.upcoming_norm = None
         x = ctx.workspace("block.x", (T, D), self.mixer.dtype)
-        if self.feed_forward is None:
+        if self.feed_forward is None or self.feed_forward_norm is None:
             self.mixer_norm.forward(ctx, h, x)
             self.mixer.forward(ctx, x, h, cache)
+            if self.feed_forward is not None:
+                self.feed_forward.forward(ctx, x, h)
         else:
             x2 = ctx.workspace("block.x2", (T, D), self.feed_forward.dtype)
             together = getattr(self.mixer_norm, "forward_with", None)

@@ -14,6 +14,14 @@ dt_bias)); S <- g S (rows); u = beta (v - S^T k); S <- S + k u^T; o = S^T q; eac
 (weight `norm` [vdim], the same for every head), times sigmoid(Wg2 Wg1 x), through Wo.  The request's state is S and
 the convolutions' last conv - 1 inputs.
 
+"mlstm"(hidden_size, heads, dim, vdim, gate_cap, eps): a matrix memory with exponential gates.  q = Wq x dim^(-1/2),
+k = Wk x [heads, dim], v = Wv x [heads, vdim]; per head the logarithms of an input and a forget gate,
+i = cap tanh((Wi x + bi) / cap), f = log sigmoid(cap tanh((Wf x + bf) / cap)); a running maximum m_t = max(f + m_(t-1), i)
+(m_0 = 0) keeps the exponentials in range: S_t = exp(f + m_(t-1) - m_t) S_(t-1) + exp(i - m_t) k v^T, n_t the same with k
+alone, o = S_t^T q / (max(|n_t . q|, exp(-m_t)) + 1e-6); each head's o is RMS-normed, the heads side by side times the
+weight `norm`, times sigmoid(Wg x), through Wo.  The request's state is S, n and m.  n is kept as one more column of S:
+the recurrence writes a 1 in the value's place there, so S^T q also yields n . q.
+
 "parallel"(hidden_size, eps, branches = [{name, mixer: PartSpec-like, out: leaf of the branch's output norm}]): every
 branch reads the same input; the result is the mean of the branches' outputs, each RMS-normed over the model width with
 a weight of its own.  The branches are mixers of any registered kind, each with the cache it asks for.
@@ -171,6 +179,72 @@ class DeltaRule(Mixer):
         ctx.note_left(h, None)
 
 
+class MLSTM(Mixer):
+    graph_safe = True
+    DEN_ADD = 1e-6          # what the read-out's denominator is enlarged by
+
+    def __init__(self, spec, dtype):
+        super().__init__(spec, dtype)
+        p = spec.params
+        self.hidden, self.heads, self.dk, self.dv = int(p["hidden_size"]), int(p["heads"]), int(p["dim"]), int(p["vdim"])
+        self.cap, self.eps = float(p["gate_cap"]), float(p["eps"])
+        if not self.cap > 0:
+            raise ValueError(f"the gates' cap must be positive, got {self.cap}")
+        leaves = _leaves({"q": "q", "k": "k", "v": "v", "gate": "g", "out": "o", "norm": "norm", "i": "i", "i_bias": "i.b", "f": "f",
+                          "f_bias": "f.b"}, p.get("names"))
+        self.names = {k: self.name(v) for k, v in leaves.items()}
+        self.qk, self.vw = self.heads * self.dk, self.heads * self.dv
+        self.cols = self.dv + 1                           # a head's columns of S: its value channels, then n
+        self.n_matrix = self.heads * self.cols * self.dk  # floats of S and n in a request's state; the maxima follow
+        self.w_in = self.w_o = self.norm = self.bias_i = self.bias_f = None
+
+    def tensors(self):
+        n, H = self.names, self.hidden
+        return {n["q"]: TensorSpec((self.qk, H)), n["k"]: TensorSpec((self.qk, H)), n["v"]: TensorSpec((self.vw, H)),
+                n["gate"]: TensorSpec((self.vw, H)), n["out"]: TensorSpec((H, self.vw)), n["norm"]: TensorSpec((self.vw,), "norm"),
+                n["i"]: TensorSpec((self.heads, H), "normal:0.0:0.1"), n["i_bias"]: TensorSpec((self.heads,), "normal:0.0:0.5"),
+                n["f"]: TensorSpec((self.heads, H), "normal:0.0:0.1"), n["f_bias"]: TensorSpec((self.heads,), "normal:3.0:1.0")}
+
+    def load(self, tensors, device):
+        n = self.names
+        get = lambda key: place(tensors[n[key]], device, self.dtype)
+        # one product for everything that reads the mixer's input, left as 32-bit sums: q | k | v | gate | i | f
+        self.w_in = torch.cat([get("q"), get("k"), get("v"), get("gate"), get("i"), get("f")], dim=0).contiguous()
+        self.w_o = get("out")
+        self.norm = place(tensors[n["norm"]], device, torch.float32)
+        self.bias_i = place(tensors[n["i_bias"]], device, torch.float32)
+        self.bias_f = place(tensors[n["f_bias"]], device, torch.float32)
+
+    def export(self):
+        n, w = self.names, self.w_in.cpu()
+        a, b, c, d, e = self.qk, 2 * self.qk, 2 * self.qk + self.vw, 2 * self.qk + 2 * self.vw, 2 * self.qk + 2 * self.vw + self.heads
+        return {n["q"]: w[:a].contiguous(), n["k"]: w[a:b].contiguous(), n["v"]: w[b:c].contiguous(), n["gate"]: w[c:d].contiguous(),
+                n["i"]: w[d:e].contiguous(), n["f"]: w[e:].contiguous(), n["out"]: self.w_o.cpu(), n["norm"]: self.norm.cpu(),
+                n["i_bias"]: self.bias_i.cpu(), n["f_bias"]: self.bias_f.cpu()}
+
+    def cache_need(self):
+        # one row per request, zero at its start: S with n as its last column [heads, vdim + 1, dim], then m [heads]
+        return FixedState((self.n_matrix + self.heads,), torch.float32)
+
+    def forward(self, ctx, x, h, cache):
+        k = kernels()
+        T, H = x.shape[0], self.heads
+        a, b, c, d = self.qk, 2 * self.qk, 2 * self.qk + self.vw, 2 * self.qk + 2 * self.vw
+        sums = ctx.workspace("linear.sums", (T, d + 2 * H), torch.float32)
+        k.gemm(x, self.w_in, sums, EPI_STORE_F32, ctx.gemm_workspace(x, self.w_in))
+        gates = ctx.workspace("mlstm.gates", (3, T, H), torch.float32)          # decay, take, floor
+        k.exp_gates(sums[:, d:d + H], sums[:, d + H:], self.bias_i, self.bias_f, self.cap, cache.state[:, self.n_matrix:],
+                    ctx.q_starts, ctx.slots, gates[0], gates[1], gates[2])
+        o = ctx.workspace("mlstm.o", (T, H * self.cols), torch.float32)
+        k.linear_scan(sums[:, :a], sums[:, a:b], sums[:, b:c], cache.state[:, :self.n_matrix], ctx.q_starts, ctx.slots, H, H,
+                      self.dk, self.cols, o, gates=(gates[0], gates[1]), v_cols=self.dv)
+        gated = ctx.workspace("linear.gated", (T, self.vw), self.dtype)
+        # (q's factor dim^(-1/2) multiplies the read-out and its normaliser alike: applied here, to both)
+        k.gated_rmsnorm(gated, o, sums[:, c:d], self.norm, self.dv, self.eps, floor=gates[2], x_scale=self.dk ** -0.5, den_add=self.DEN_ADD)
+        k.gemm(gated, self.w_o, h, EPI_ACCUM_F32, ctx.gemm_workspace(gated, self.w_o))
+        ctx.note_left(h, None)
+
+
 class Parallel(Mixer):
     """Branches side by side on the same input; h += mean_b rmsnorm(branch_b(x)) * out_b."""
 
@@ -243,4 +317,5 @@ class Parallel(Mixer):
 
 register_mixer("lightning", Lightning)
 register_mixer("delta_rule", DeltaRule)
+register_mixer("mlstm", MLSTM)
 register_mixer("parallel", Parallel)

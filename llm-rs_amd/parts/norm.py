@@ -145,3 +145,34 @@ class DynamicTanh(Norm):
 
 
 register_norm("dyt", DynamicTanh)
+
+
+class LayerNorm(Norm):
+    """Layer norm(size, eps) with weight and bias: y = (x - mean) / sqrt(var + eps) * weight + bias, var the mean of the
+    squared deviations from the mean.  32-bit throughout, one rounding on the way out.  Tensors: the weight under the
+    prefix itself, the bias under `<prefix>.b` (`names` gives other leaves)."""
+    graph_safe = True
+
+    def __init__(self, spec, dtype):
+        super().__init__(spec, dtype)
+        self.size = int(spec.params["size"])
+        self.eps = float(spec.params["eps"])
+        leaves = {"weight": "", "bias": "b", **(spec.params.get("names") or {})}
+        self.names = {key: (self.name(leaf) if leaf else self.prefix) for key, leaf in leaves.items()}
+        self.weight = self.bias = None
+
+    def tensors(self):
+        return {self.names["weight"]: TensorSpec((self.size,), "norm"), self.names["bias"]: TensorSpec((self.size,), "normal:0.0:0.1")}
+
+    def load(self, tensors, device):
+        self.weight = place(tensors[self.names["weight"]], device, torch.float32)
+        self.bias = place(tensors[self.names["bias"]], device, torch.float32)
+
+    def export(self):
+        return {self.names["weight"]: self.weight.cpu(), self.names["bias"]: self.bias.cpu()}
+
+    def forward(self, ctx, h, out, rows=None):
+        kernels().layernorm(out, h, self.weight, self.bias, self.eps, rows)
+
+
+register_norm("layernorm", LayerNorm)
