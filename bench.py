@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Decode and prefill throughput of the engine on one MI355X.
 
-    python bench.py --gpus 1 --steps K --warmup W [--workload decode8b|serve1b|mixed70b|sizes|sizes1b|prompts|long|widths|portions|tuvodra|lilatar|vivisun]
+    python bench.py --gpus 1 --steps K --warmup W [--workload decode8b|serve1b|mixed70b|sizes|sizes1b|prompts|long|widths|portions|tuvodra|lilatar|vivisun|gokosun]
 
 The default run (`decode8b`) is the Llama-3.1-8B shape with random bfloat16 weights: 8
 requests, each with 2,048 tokens of context in the cache, decode K steps through the
@@ -39,6 +39,10 @@ The other workloads print one line of the same form each:
             dense and routed squared-relu feed-forwards).
   vivisun   the same for the Vivisun decoder (dynamic-tanh norms, both halves of a layer on the same stream; attention
             with convolved q/k/v, normed and half-rotated heads and a gate, in turns with latent attention with a sink).
+  gokosun   the same for the Gokosun decoder (one layer norm for both halves of a layer; latent attention with a query
+            latent, a rotated key part and a sink, grouped-query attention with mixed values, a matrix memory with
+            exponential gates, in threes; clamped gated feed-forwards, dense and as sigmoid-routed experts beside a
+            shared one).
 With LLM_PERF set in the environment every kernel call is timed by itself and a table
 by kernel goes to stderr (the reference's switch, src/backend/metal/mod.rs:235,321-400).
 """
@@ -69,7 +73,7 @@ LLAMA_8B = _llama(32, 4096, 32, 8, 128, 14336, 8.0, False)
 LLAMA_1B = _llama(16, 2048, 32, 8, 64, 8192, 32.0, True)
 LLAMA_70B = _llama(80, 8192, 64, 8, 128, 28672, 8.0, False)
 SHAPES = {"Llama-3.1-8B shape": LLAMA_8B, "Llama-3.2-1B shape": LLAMA_1B, "Llama-3.1-70B shape": LLAMA_70B}
-WORKLOADS = ("decode8b", "serve1b", "mixed70b", "sizes", "sizes1b", "prompts", "long", "widths", "portions", "tuvodra", "lilatar", "vivisun")
+WORKLOADS = ("decode8b", "serve1b", "mixed70b", "sizes", "sizes1b", "prompts", "long", "widths", "portions", "tuvodra", "lilatar", "vivisun", "gokosun")
 
 
 def flat_config(model: str, layers_run: int, global_batch: int, seq_len: int, page_size: int, **more) -> dict:
@@ -696,6 +700,48 @@ def run_vivisun(args) -> dict:
     return line
 
 
+def gokosun_shape(width, heads, kv_heads, dim, ff, kv_rank, repeats, experts, top, vocab=128256):
+    """Layers in threes: latent attention (the Llama shape's heads with `dim` unrotated and dim / 2 rotated features,
+    queries through a vector of width / 2, keys and values from one of kv_rank less the rotated part, so that a token
+    leaves kv_rank numbers in the cache) with the Llama shape's feed-forward; grouped-query attention with the Llama
+    shape's heads, all of a head rotated, values mixed with the first such layer's, and experts of which the chosen ones
+    and the shared one are together as wide as the dense feed-forward; a matrix memory with heads of 64 key and 128 value
+    channels, as wide as the stream, with the dense feed-forward."""
+    rot = dim // 2
+    part = ff // (top + 1)
+    three = [{"type": "latent_attention",
+              "mixer": {"heads": heads, "dim": dim, "rot_dim": rot, "vdim": dim, "kv_rank": kv_rank - rot, "q_rank": width // 2, "scale": (dim + rot) ** -0.5,
+                        "rot": {"dims": rot, "base": 500000.0, "scaling": {"factor": 8.0, "original": 8192, "fast": 32.0, "slow": 1.0}}},
+              "mlp": {"kind": "dense", "ff": ff, "limit": 7.0}},
+             {"type": "attention", "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5, "v_mix": True,
+                                             "rot": {"dims": dim, "base": 500000.0}},
+              "mlp": {"kind": "moe", "expert": {"ff": part, "limit": 7.0}, "router": {"experts": experts, "top": top, "scale": 2.5},
+                      "shared": {"ff": part, "limit": 7.0}}},
+             {"type": "mlstm", "mixer": {"heads": width // 128, "dim": 64, "vdim": 128, "gate_cap": 15.0}, "mlp": {"kind": "dense", "ff": ff, "limit": 7.0}}]
+    import copy
+    return {"architecture": "Gokosun", "vocab": vocab, "width": width, "norm": {"eps": 1e-6},
+            "layers": [copy.deepcopy(l) for _ in range(repeats) for l in three]}
+
+
+def run_gokosun(args) -> dict:
+    """Prompt and decode throughput of the Gokosun decoder at two widths, each beside a Llama decoder of the same
+    width, heads, feed-forward and number of layers (random weights both)."""
+    repeats = max(1, (args.layers or 6) // 3)
+    sizes = {"1B widths": (LLAMA_1B, 2048, 32, 8, 64, 8192), "8B widths": (LLAMA_8B, 4096, 32, 8, 128, 14336)}
+    pairs = {size: {"gokosun": gokosun_shape(width, heads, kv_heads, dim, ff, args.kv_rank, repeats, args.experts, args.top),
+                    "llama": dict(llama, num_hidden_layers=3 * repeats)}
+             for size, (llama, width, heads, kv_heads, dim, ff) in sizes.items()}
+    points = run_beside_llama(args, pairs, 3 * repeats)
+    first = next(iter(points.values()))
+    line = base_line("decode_tokens_per_s", first["decode_tokens_per_s"], args.steps, args.warmup, first["decode_ms_per_step"] * 1e-3, args.dtype,
+                     {"model": "Gokosun (latent attention with a query latent, a rotated key part and a sink + dense feed-forward; grouped-query attention "
+                               "with mixed values + experts; a matrix memory with exponential gates + dense feed-forward; in threes) beside Llama of equal widths",
+                      "global_batch": args.batch, "seq_len": args.context, "parallelism": "single GPU", "layers_run": 3 * repeats,
+                      "prefill_tokens": args.prefill_tokens, "kv_rank": args.kv_rank, "experts": args.experts, "top": args.top, "page_size": 16})
+    line["points"] = points
+    return line
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -714,11 +760,11 @@ def main() -> int:
     ap.add_argument("--new-tokens", type=int, default=256, help="serve1b: tokens generated for each request")
     ap.add_argument("--max-batch-tokens", type=int, default=2048, help="serve1b: tokens a scheduler step may run")
     ap.add_argument("--window", type=int, default=1024, help="tuvodra, lilatar: keys an attention layer sees")
-    ap.add_argument("--only-size", default="", help="tuvodra, lilatar, vivisun: run one of the sizes only (1B or 8B)")
-    ap.add_argument("--kv-rank", type=int, default=256, help="vivisun: width of the latent vector a token leaves in the cache")
+    ap.add_argument("--only-size", default="", help="tuvodra, lilatar, vivisun, gokosun: run one of the sizes only (1B or 8B)")
+    ap.add_argument("--kv-rank", type=int, default=256, help="vivisun, gokosun: how many numbers a token of a latent layer leaves in the cache")
     ap.add_argument("--loop-times", type=int, default=1, help="vivisun: how often the layers after the first run in a row")
-    ap.add_argument("--experts", type=int, default=16, help="lilatar: experts of a routed feed-forward")
-    ap.add_argument("--top", type=int, default=4, help="lilatar: experts a token uses")
+    ap.add_argument("--experts", type=int, default=16, help="lilatar, gokosun: experts of a routed feed-forward")
+    ap.add_argument("--top", type=int, default=4, help="lilatar, gokosun: experts a token uses")
     ap.add_argument("--experts-by-rows-from", type=int, default=None,
                     help="lilatar: rows an expert gets on average from which a prompt step runs the experts one by one (default: the part's own rule)")
     args = ap.parse_args()
@@ -730,7 +776,7 @@ def main() -> int:
     args.warmup = args.warmup if args.warmup is not None else (2 if heavy else 8)
     line = {"decode8b": run_decode8b, "serve1b": run_serve1b, "mixed70b": run_mixed70b, "sizes": run_sizes, "sizes1b": run_sizes,
             "prompts": run_prompts, "long": run_long, "widths": run_widths, "portions": run_portions, "tuvodra": run_tuvodra, "lilatar": run_lilatar,
-            "vivisun": run_vivisun}[args.workload](args)
+            "vivisun": run_vivisun, "gokosun": run_gokosun}[args.workload](args)
     from llm_rs_amd.kernels import kernels
     if kernels().times is not None:         # LLM_PERF: what was still to be shown of the per-kernel table
         kernels().times.dump()

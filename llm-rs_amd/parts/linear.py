@@ -224,7 +224,8 @@ class MLSTM(Mixer):
 
     def cache_need(self):
         # one row per request, zero at its start: S with n as its last column [heads, vdim + 1, dim], then m [heads]
-        return FixedState((self.n_matrix + self.heads,), torch.float32)
+        # (in room for a multiple of four, so that a slot's rows stay whole 16-byte pieces where S's are)
+        return FixedState((self.n_matrix + -(-self.heads // 4) * 4,), torch.float32)
 
     def forward(self, ctx, x, h, cache):
         k = kernels()

@@ -39,17 +39,57 @@ class EmulatedKernels(Kernels):
         g = torch.sigmoid(gate).repeat_interleave(per, dim=1)
         o.copy_((o.float() * g).to(o.dtype))
 
-    def latent_finish(self, sums, q, q_size, rank, weight, eps, slot_map, k_cache, v_cache, page_size, num_pages, write):
-        q.copy_(sums[:, :q_size].to(q.dtype))
+    def layernorm(self, out, x, weight, bias, eps, rows=None):
+        src = x if rows is None else x[rows.long()]
+        dev = src - src.mean(-1, keepdim=True)
+        out.copy_((dev / torch.sqrt((dev * dev).mean(-1, keepdim=True) + eps) * weight + bias).to(out.dtype))
+
+    def latent_finish(self, sums, q, q_size, rank, weight, eps, slot_map, k_cache, v_cache, page_size, num_pages, write,
+                      q_weight=None, rotated=None):
+        first = sums[:, :q_size]
+        if q_weight is not None:
+            first = first / torch.sqrt((first * first).mean(-1, keepdim=True) + eps) * q_weight
+        q.copy_(first.to(q.dtype))
         if not write:
             return
         c = sums[:, q_size:q_size + rank]
         c = c / torch.sqrt((c * c).mean(-1, keepdim=True) + eps) * weight
-        kc, vc = k_cache.view(num_pages, page_size, rank), v_cache.view(num_pages, rank, page_size)
+        if rotated is not None:
+            rot, positions, inv_freq, gain = rotated
+            part = sums[:, q_size + rank:q_size + rank + rot].clone()
+            angle = positions.float()[:, None] * inv_freq[None, :]
+            cos, sin = torch.cos(angle) * gain, torch.sin(angle) * gain
+            a, b = part[:, 0::2].clone(), part[:, 1::2].clone()
+            part[:, 0::2], part[:, 1::2] = a * cos - b * sin, b * cos + a * sin
+            c = torch.cat([c, part], dim=1)
+        width = c.shape[1]
+        kc, vc = k_cache.view(num_pages, page_size, width), v_cache.view(num_pages, width, page_size)
         page, off = (slot_map // page_size).long(), (slot_map % page_size).long()
         for t in range(sums.shape[0]):
             kc[page[t], off[t], :] = c[t].to(kc.dtype)
             vc[page[t], :, off[t]] = c[t].to(vc.dtype)
+
+    def qkv_whole(self, sums, q_cols, k_cols, v_cols, q_weight, k_weight, eps, first=None, lam=None, keep=None):
+        for w, lo, n in ((q_weight, 0, q_cols), (k_weight, q_cols, k_cols)):
+            if w is not None:
+                x = sums[:, lo:lo + n]
+                x.copy_(x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * w)
+        v = sums[:, q_cols + k_cols:q_cols + k_cols + v_cols]
+        if first is not None:
+            v.copy_((1.0 - lam) * v + lam * first)
+        elif keep is not None:
+            keep.copy_(v)
+
+    def exp_gates(self, gi, gf, bias_i, bias_f, cap, m_state, q_starts, slots, decay, take, floor):
+        i = cap * torch.tanh((gi + (bias_i if bias_i is not None else 0.0)) / cap)
+        f = torch.nn.functional.logsigmoid(cap * torch.tanh((gf + (bias_f if bias_f is not None else 0.0)) / cap))
+        H = gi.shape[1]
+        for e in range(slots.numel()):
+            m = m_state[int(slots[e])][:H]
+            for t in range(int(q_starts[e]), int(q_starts[e + 1])):
+                m_new = torch.maximum(f[t] + m, i[t])
+                decay[t], take[t], floor[t] = torch.exp(f[t] + m - m_new), torch.exp(i[t] - m_new), torch.exp(-m_new)
+                m.copy_(m_new)
 
     def head_product(self, a, w, out, gate=None):
         H, n_out, n_in = w.shape
@@ -257,8 +297,11 @@ class EmulatedKernels(Kernels):
         a.copy_(torch.exp(-torch.exp(A_log)[None, :, None] * soft).reshape(T, -1))
         b.copy_(1.0 / (1.0 + torch.exp(-b)))
 
-    def linear_scan(self, q, k, v, state, q_starts, slots, heads, qk_heads, dk, dv, out, decay=None, g=None, beta=None):
+    def linear_scan(self, q, k, v, state, q_starts, slots, heads, qk_heads, dk, dv, out, decay=None, g=None, beta=None, gates=None,
+                    v_cols=0):
         rep = heads // qk_heads
+        if v_cols and v_cols < dv:          # the columns past v's own are written with 1
+            v = torch.cat([v.view(-1, heads, v_cols), torch.ones(v.shape[0], heads, dv - v_cols, dtype=v.dtype)], dim=2).reshape(v.shape[0], -1)
         for e in range(slots.numel()):
             S = state[int(slots[e])][:heads * dk * dv].view(heads, dv, dk).transpose(1, 2)       # kept value channel by key channel
             for t in range(int(q_starts[e]), int(q_starts[e + 1])):
@@ -269,12 +312,19 @@ class EmulatedKernels(Kernels):
                     S.mul_(g[t].view(heads, dk)[:, :, None])
                 elif decay is not None:
                     S.mul_(decay[:, None, None])
+                elif gates is not None:
+                    S.mul_(gates[0][t][:, None, None])
+                    vt = vt * gates[1][t][:, None]
                 u = vt if beta is None else beta[t][:, None] * (vt - torch.einsum("hkv,hk->hv", S, kt))
                 S.add_(kt[:, :, None] * u[:, None, :])
                 out[t] = torch.einsum("hkv,hk->hv", S, qt).reshape(-1)
 
-    def gated_rmsnorm(self, out, x, gate, weight, group, eps):
-        T, W = x.shape
+    def gated_rmsnorm(self, out, x, gate, weight, group, eps, floor=None, x_scale=1.0, den_add=0.0):
+        T, W = gate.shape
+        if floor is not None:
+            wide = x.reshape(T, W // group, group + 1)
+            den = torch.maximum(wide[:, :, group].abs() * x_scale, floor) + den_add
+            x = (wide[:, :, :group] * x_scale / den[:, :, None]).reshape(T, W)
         parts = x.reshape(T, W // group, group)
         y = (parts / torch.sqrt((parts * parts).mean(-1, keepdim=True) + eps)).reshape(T, W)
         w = weight if weight.numel() == W else weight.repeat(W // group)
@@ -285,17 +335,22 @@ class EmulatedKernels(Kernels):
             v = x if bias is None else x + bias
             out.add_(coef * v / torch.sqrt((v * v).mean(-1, keepdim=True) + eps) * weight)
 
-    def route_topk(self, logits, weights, top, renormalize=False):
-        scores = torch.softmax(logits, dim=-1)
+    def route_topk(self, logits, weights, top, renormalize=False, score="softmax", correction=None, scale=1.0):
+        scores = torch.softmax(logits, dim=-1) if score == "softmax" else torch.sigmoid(logits)
+        choice = scores if correction is None else scores + correction
         weights.zero_()
         for t in range(logits.shape[0]):
-            chosen = sorted(range(logits.shape[1]), key=lambda e: (-float(scores[t, e]), e))[:top]
-            total = sum(float(scores[t, e]) for e in chosen) if renormalize else 1.0
+            chosen = sorted(range(logits.shape[1]), key=lambda e: (-float(choice[t, e]), e))[:top]
+            total = (sum(float(scores[t, e]) for e in chosen) + (1e-20 if score == "sigmoid" else 0.0)) if renormalize else 1.0
             for e in chosen:
-                weights[t, e] = scores[t, e] / total
+                weights[t, e] = scores[t, e] / total * scale
 
-    def act_weight(self, out, up, weights, ff):
-        y = torch.clamp(up, min=0.0) ** 2
+    def act_weight(self, out, up, weights, ff, activation="relu2", limit=0.0, alpha=1.0):
+        if activation == "clamped_glu":
+            g, u = torch.clamp(up[:, 0::2], max=limit), torch.clamp(up[:, 1::2], min=-limit, max=limit)
+            y = g * torch.sigmoid(alpha * g) * (u + 1.0)
+        else:
+            y = torch.clamp(up, min=0.0) ** 2
         if weights is not None:
             y = y * weights.repeat_interleave(ff, dim=1)
         out.copy_(y.to(out.dtype))
