@@ -708,7 +708,7 @@ def gokosun_shape(width, heads, kv_heads, dim, ff, kv_rank, repeats, experts, to
     and the shared one are together as wide as the dense feed-forward; a matrix memory with heads of 64 key and 128 value
     channels, as wide as the stream, with the dense feed-forward."""
     rot = dim // 2
-    part = ff // (top + 1)
+    part = max(128, ff // (top + 1) // 128 * 128)
     three = [{"type": "latent_attention",
               "mixer": {"heads": heads, "dim": dim, "rot_dim": rot, "vdim": dim, "kv_rank": kv_rank - rot, "q_rank": width // 2, "scale": (dim + rot) ** -0.5,
                         "rot": {"dims": rot, "base": 500000.0, "scaling": {"factor": 8.0, "original": 8192, "fast": 32.0, "slow": 1.0}}},

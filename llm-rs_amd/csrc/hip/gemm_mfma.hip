@@ -53,6 +53,14 @@ __device__ __forceinline__ float swap_neighbours(float x) {
 __device__ __forceinline__ float silu_fast_f32(float x) {
     return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * -1.44269504088896341f));
 }
+// act(gate, up) of the two gated epilogues with the same instructions
+__device__ __forceinline__ float gated_act_fast(int epi, float g, float u) {
+    if (epi == LLMRS_EPI_SWIGLU) return silu_fast_f32(g) * u;
+    const float limit = llmrs_glu_clamp.limit;
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g * (llmrs_glu_clamp.alpha * -1.44269504088896341f))) * (u + 1.0f);
+}
 
 // The tile loops' barrier: this wave's LDS reads and writes are done, then every wave of the block
 // has arrived.  Unlike __syncthreads() it does not wait for loads from memory that are still in
@@ -240,10 +248,10 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __rest
 #pragma unroll
             for (int r = 0; r < 4; ++r)
                 if (n + r < N) partial[((size_t)blockIdx.y * M + m) * N + n + r] = v[r];
-        } else if (epi == LLMRS_EPI_SWIGLU) {
+        } else if (epi_gated(epi)) {
 #pragma unroll
             for (int r = 0; r < 4; r += 2)
-                if (n + r + 1 < N) ((bf16*)out)[(size_t)m * ldc + (n + r) / 2] = (bf16)(silu_f32(v[r]) * v[r + 1]);
+                if (n + r + 1 < N) ((bf16*)out)[(size_t)m * ldc + (n + r) / 2] = (bf16)gated_act(epi, v[r], v[r + 1]);
         } else if (epi == LLMRS_EPI_QKV) {
             // four consecutive features of one head: two rotation pairs (2i, 2i+1); the
             // rotation is applied to the 32-bit sums, which are rounded once
@@ -334,8 +342,8 @@ __global__ void gemm_splitk_finish_kernel(const float* __restrict__ partial, int
         v0 += p[0];
         if (has1) v1 += p[1];
     }
-    if (epi == LLMRS_EPI_SWIGLU) {
-        if (has1) ((bf16*)out)[(size_t)m * ldc + n / 2] = (bf16)(silu_f32(v0) * v1);
+    if (epi_gated(epi)) {
+        if (has1) ((bf16*)out)[(size_t)m * ldc + n / 2] = (bf16)gated_act(epi, v0, v1);
     } else {
         epilogue_store<bf16>(epi, out, ldc, m, n, v0);
         if (has1) epilogue_store<bf16>(epi, out, ldc, m, n + 1, v1);
@@ -524,10 +532,10 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
         for (int r = 0; r < 16; ++r) {
             int m = m0 + wm * TM + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
             float v = acc[i][j][r];
-            if (epi == LLMRS_EPI_SWIGLU) {
+            if (epi_gated(epi)) {
                 float other = __shfl_xor(v, 1, 64);   // even lane: gate here, up next door
                 if (!(lane & 1) && m < M && n + 1 < N)
-                    ((bf16*)out)[(size_t)m * ldc + n / 2] = (bf16)(silu_f32(v) * other);
+                    ((bf16*)out)[(size_t)m * ldc + n / 2] = (bf16)gated_act(epi, v, other);
             } else if (m < M && n < N) {
                 epilogue_store<bf16>(epi, out, ldc, m, n, v);
             }
@@ -607,10 +615,10 @@ __device__ __forceinline__ void tile_epilogue(f32x16 (&acc)[BM / WGM / 32][BN / 
     // 16-bit results: a lane holds one column of 16 rows, which stored as they lie would be 2 bytes
     // per lane and store.  The wave puts its tile through LDS (free after the loop's last barrier; each
     // wave has room for its own tile) and stores it row by row, 16 bytes per lane, whole lines at a time.
-    bool staged = (epi == LLMRS_EPI_STORE || epi == LLMRS_EPI_SWIGLU) && ldc % 8 == 0 && ((uintptr_t)out & 15) == 0 &&
-                  (epi == LLMRS_EPI_SWIGLU ? N % 16 == 0 : N % 8 == 0);
+    bool staged = (epi == LLMRS_EPI_STORE || epi_gated(epi)) && ldc % 8 == 0 && ((uintptr_t)out & 15) == 0 &&
+                  (epi_gated(epi) ? N % 16 == 0 : N % 8 == 0);
     if (staged) {
-        const bool glu = epi == LLMRS_EPI_SWIGLU;
+        const bool glu = epi_gated(epi);
         const int cols = glu ? TN / 2 : TN;                       // columns of the wave's tile as stored
         const int row_bytes = cols * 2;
         static_assert(TN * 2 * TM * WAVES <= SMEM_BYTES, "the waves' tiles must fit in the tile buffers");
@@ -630,7 +638,7 @@ __device__ __forceinline__ void tile_epilogue(f32x16 (&acc)[BM / WGM / 32][BN / 
                 float v0 = acc[i][j][r], v1 = acc[i][j][r + 1];
                 float got = swap_neighbours(odd ? v0 : v1);
                 float left = odd ? got : v0, right = odd ? v1 : got;       // columns c & ~1 and c | 1 of `row`
-                if (glu) *(bf16*)(mine + row * row_bytes + (c / 2) * 2) = (bf16)(silu_fast_f32(left) * right);
+                if (glu) *(bf16*)(mine + row * row_bytes + (c / 2) * 2) = (bf16)gated_act_fast(epi, left, right);
                 else {
                     bf16x2 two;
                     two[0] = (bf16)left;
@@ -657,10 +665,10 @@ __device__ __forceinline__ void tile_epilogue(f32x16 (&acc)[BM / WGM / 32][BN / 
         for (int r = 0; r < 16; ++r) {
             int m = m0 + wm * TM + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
             float v = acc[i][j][r];
-            if (epi == LLMRS_EPI_SWIGLU) {
+            if (epi_gated(epi)) {
                 float other = __shfl_xor(v, 1, 64);
                 if (!(lane & 1) && m < M && n + 1 < N)
-                    ((bf16*)out)[(size_t)m * ldc + n / 2] = (bf16)(silu_f32(v) * other);
+                    ((bf16*)out)[(size_t)m * ldc + n / 2] = (bf16)gated_act(epi, v, other);
             } else if (m < M && n < N) {
                 epilogue_store<bf16>(epi, out, ldc, m, n, v);
             }
@@ -1025,7 +1033,7 @@ __device__ __forceinline__ void band_epilogue(f32x16 (&acc)[BM / 64][BN / 64], u
             __builtin_amdgcn_sched_barrier(0);       // one part of the tile at a time: its old values are not asked for earlier
         });
     } else {
-        constexpr bool glu = EPI == LLMRS_EPI_SWIGLU;
+        constexpr bool glu = EPI == LLMRS_EPI_SWIGLU || EPI == LLMRS_EPI_GLU_CLAMP;
         constexpr int cols = glu ? TN / 2 : TN;      // columns of the wave's band as stored
         constexpr int row_bytes = cols * 2;
         unsigned char* mine = smem + wave * (32 * TN * 2);
@@ -1043,7 +1051,7 @@ __device__ __forceinline__ void band_epilogue(f32x16 (&acc)[BM / 64][BN / 64], u
                     float v0 = acc[i][j][r], v1 = acc[i][j][r + 1];
                     float got = swap_neighbours(odd ? v0 : v1);
                     float left = odd ? got : v0, right = odd ? v1 : got;
-                    if (glu) *(bf16*)(mine + row * row_bytes + (cc / 2) * 2) = (bf16)(silu_fast_f32(left) * right);
+                    if (glu) *(bf16*)(mine + row * row_bytes + (cc / 2) * 2) = (bf16)gated_act_fast(EPI, left, right);
                     else {
                         bf16x2 two;
                         two[0] = (bf16)left;
@@ -1210,7 +1218,7 @@ __global__ __launch_bounds__(256) void gemm_fourwave_kernel(const bf16* __restri
 static bool fourwave_takes(int epi, const void* out, int ldc, int N) {
     if (epi == LLMRS_EPI_ACCUM_F32 || epi == LLMRS_EPI_STORE_F32) return true;
     if (epi == LLMRS_EPI_STORE) return ldc % 8 == 0 && ((uintptr_t)out & 15) == 0 && N % 8 == 0;
-    if (epi == LLMRS_EPI_SWIGLU) return ldc % 8 == 0 && ((uintptr_t)out & 15) == 0 && N % 16 == 0;
+    if (epi_gated(epi)) return ldc % 8 == 0 && ((uintptr_t)out & 15) == 0 && N % 16 == 0;
     return false;
 }
 template <int BM, int BN, int EPI>
@@ -1236,6 +1244,7 @@ static int launch_fourwave(hipStream_t stream, const bf16* A, int lda, const bf1
         case LLMRS_EPI_STORE_F32: return launch_fourwave_epi<BM, BN, LLMRS_EPI_STORE_F32>(stream, A, lda, W, out, ldc, M, N, K);
         case LLMRS_EPI_ACCUM_F32: return launch_fourwave_epi<BM, BN, LLMRS_EPI_ACCUM_F32>(stream, A, lda, W, out, ldc, M, N, K);
         case LLMRS_EPI_SWIGLU: return launch_fourwave_epi<BM, BN, LLMRS_EPI_SWIGLU>(stream, A, lda, W, out, ldc, M, N, K);
+        case LLMRS_EPI_GLU_CLAMP: return launch_fourwave_epi<BM, BN, LLMRS_EPI_GLU_CLAMP>(stream, A, lda, W, out, ldc, M, N, K);
         default: return llmrs_fail("gemm: the four-wave tiles have no epilogue %d", epi);
     }
 }
@@ -1354,11 +1363,12 @@ int llmrs_gemm_bf16_split_parts(hipStream_t stream, const bf16* A, int lda, cons
 
 int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16* W, void* out, int ldc,
                          int M, int N, int K, int epi, void* workspace, size_t workspace_bytes,
-                         const QkvEpilogue* qkv, const RowScale* scale, const NextNorm* next) {
+                         const QkvEpilogue* qkv, const RowScale* scale, const NextNorm* next, const GluClamp* glu) {
     if (K % 8 || lda % 8 || ((uintptr_t)A & 15) || ((uintptr_t)W & 15)) {
         if (scale != nullptr || next != nullptr) { llmrs_fail("gemm: a deferred norm needs rows of a multiple of 8 values, 16-byte aligned"); return -1; }
         return 0;
     }
+    if (glu != nullptr) glu_clamp_set(stream, *glu);      // (a call that hands part of its rows on to itself has set them already)
     const bool whole = next != nullptr && next->eps > 0.0f;      // the norm that follows is finished by the kernel that adds the parts up
     if (whole) {
         bool ok = scale == nullptr && epi == LLMRS_EPI_ACCUM_F32 && llmrs_gemm_norms_whole(M, N, K) && workspace != nullptr &&
@@ -1505,7 +1515,7 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
             bool split_pays = (double)(whole / cus) + 0.62 * ceil_div(small_blocks, 2L * cus) < (double)ceil_div(big_tiles, (long)cus);
             if (n_split > 0 && n_split < N && rest > 0 && 2 * rest <= cus + cus / 4 && split_pays) {
                 size_t elt = (epi == LLMRS_EPI_STORE_F32 || epi == LLMRS_EPI_ACCUM_F32) ? sizeof(float) : sizeof(bf16);
-                void* out_rest = (char*)out + (size_t)(epi == LLMRS_EPI_SWIGLU ? n_split / 2 : n_split) * elt;
+                void* out_rest = (char*)out + (size_t)(epi_gated(epi) ? n_split / 2 : n_split) * elt;
                 rc = four && fourwave_takes(epi, out, ldc, n_split)
                          ? launch_fourwave<256, 256>(stream, A, lda, W, out, ldc, M, n_split, K, epi)
                      : small ? launch_pingpong<256, 256, 2, 4, true>(stream, A, lda, W, out, ldc, M, n_split, K, epi)

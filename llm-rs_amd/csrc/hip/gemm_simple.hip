@@ -49,11 +49,11 @@ __global__ __launch_bounds__(256) void gemm_simple_kernel(const T* __restrict__ 
     for (int i = 0; i < 4; ++i) {
         int m = m0 + ty * 4 + i;
         if (m >= M) continue;
-        if (epi == LLMRS_EPI_SWIGLU) {
+        if (epi_gated(epi)) {
 #pragma unroll
             for (int j = 0; j < 4; j += 2) {
                 int n = n0 + tx * 4 + j;
-                if (n + 1 < N) ((T*)out)[(size_t)m * ldc + n / 2] = from_f32<T>(silu_f32(acc[i][j]) * acc[i][j + 1]);
+                if (n + 1 < N) ((T*)out)[(size_t)m * ldc + n / 2] = from_f32<T>(gated_act(epi, acc[i][j], acc[i][j + 1]));
             }
         } else {
 #pragma unroll
@@ -160,10 +160,10 @@ __global__ __launch_bounds__(256) void gemm_f32_mfma_kernel(const float* __restr
             for (int r = 0; r < 16; ++r) {
                 int m = m0 + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
                 float v = acc[i][j][r];
-                if (epi == LLMRS_EPI_SWIGLU) {
+                if (epi_gated(epi)) {
                     float other = __shfl_xor(v, 1, 64);   // even lane: gate here, up next door
                     if (!(lane & 1) && m < M && n + 1 < N)
-                        ((float*)out)[(size_t)m * ldc + n / 2] = silu_f32(v) * other;
+                        ((float*)out)[(size_t)m * ldc + n / 2] = gated_act(epi, v, other);
                 } else if (m < M && n < N) {
                     epilogue_store<float>(epi, out, ldc, m, n, v);
                 }
@@ -226,8 +226,8 @@ __global__ __launch_bounds__(256) void gemm_rows_kernel(const T* __restrict__ A,
         if (lane != 0) continue;
 #pragma unroll
         for (int r = 0; r < RW; r += 2) {
-            if (epi == LLMRS_EPI_SWIGLU) {
-                if (n + r + 1 < N) ((T*)out)[(size_t)m * ldc + (n + r) / 2] = from_f32<T>(silu_f32(v[r]) * v[r + 1]);
+            if (epi_gated(epi)) {
+                if (n + r + 1 < N) ((T*)out)[(size_t)m * ldc + (n + r) / 2] = from_f32<T>(gated_act(epi, v[r], v[r + 1]));
             } else {
                 if (n + r < N) epilogue_store<T>(epi, out, ldc, m, n + r, v[r]);
                 if (n + r + 1 < N) epilogue_store<T>(epi, out, ldc, m, n + r + 1, v[r + 1]);
@@ -312,10 +312,10 @@ __global__ __launch_bounds__(NW * 64) void gemm_f32_skinny_kernel(const float* _
         }
         int m = row, n = n0 + nt * 16 + 4 * g;
         if (m >= M) continue;
-        if (epi == LLMRS_EPI_SWIGLU) {
+        if (epi_gated(epi)) {
 #pragma unroll
             for (int r = 0; r < 4; r += 2)
-                if (n + r + 1 < N) ((float*)out)[(size_t)m * ldc + (n + r) / 2] = silu_f32(v[r]) * v[r + 1];
+                if (n + r + 1 < N) ((float*)out)[(size_t)m * ldc + (n + r) / 2] = gated_act(epi, v[r], v[r + 1]);
         } else {
 #pragma unroll
             for (int r = 0; r < 4; ++r)
@@ -346,11 +346,13 @@ static void launch_f32_skinny(hipStream_t stream, const float* A, int lda, const
 extern "C" int llmrs_gemm(hipStream_t stream, int dtype, const void* A, int lda, const void* W, void* out, int ldc,
                           int M, int N, int K, int epi, void* workspace, size_t workspace_bytes, int allow_mfma,
                           const float* scale_sumsq, int scale_parts, float scale_eps, float* next_sumsq, void* next_y,
-                          int next_ldy, const float* next_weight, float next_eps) {
+                          int next_ldy, const float* next_weight, float next_eps, float glu_limit, float glu_alpha) {
     LLMRS_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
     LLMRS_REQUIRE(lda >= K, "gemm: row stride %d of A is shorter than K=%d", lda, K);
-    LLMRS_REQUIRE(epi >= 0 && epi <= 3, "gemm: unknown epilogue %d", epi);
-    if (epi == LLMRS_EPI_SWIGLU) {
+    LLMRS_REQUIRE((epi >= 0 && epi <= 3) || epi == LLMRS_EPI_GLU_CLAMP, "gemm: unknown epilogue %d", epi);
+    LLMRS_REQUIRE(epi != LLMRS_EPI_GLU_CLAMP || glu_limit > 0.0f, "gemm: the clamped gated epilogue needs a positive limit, got %g", glu_limit);
+    const GluClamp glu{glu_limit, glu_alpha};
+    if (epi_gated(epi)) {
         LLMRS_REQUIRE(N % 2 == 0, "gemm: the gate/up epilogue needs an even N, got %d", N);
         LLMRS_REQUIRE(ldc >= N / 2, "gemm: row stride %d of out is shorter than N/2=%d", ldc, N / 2);
     } else {
@@ -361,9 +363,11 @@ extern "C" int llmrs_gemm(hipStream_t stream, int dtype, const void* A, int lda,
         RowScale rs{scale_sumsq, scale_parts, scale_eps};
         NextNorm nn{next_sumsq, (bf16*)next_y, next_ldy, next_weight, next_eps};
         int took = llmrs_gemm_bf16_mfma(stream, (const bf16*)A, lda, (const bf16*)W, out, ldc, M, N, K, epi, workspace,
-                                        workspace_bytes, nullptr, scale_sumsq ? &rs : nullptr, next_y ? &nn : nullptr);
+                                        workspace_bytes, nullptr, scale_sumsq ? &rs : nullptr, next_y ? &nn : nullptr,
+                                        epi == LLMRS_EPI_GLU_CLAMP ? &glu : nullptr);
         if (took != 0) return took < 0 ? -1 : 0;
     }
+    if (epi == LLMRS_EPI_GLU_CLAMP) glu_clamp_set(stream, glu);       // (this source file's kernels read their own variable)
     LLMRS_REQUIRE(scale_sumsq == nullptr && next_y == nullptr, "gemm: a deferred norm needs the bfloat16 matrix-core kernels (M=%d N=%d K=%d)", M, N, K);
     // (one or two tokens are better off with the walk below, which then asks for little beside the weights:
     // a decode step of the 8B shape at one request 7.1 against 7.8 ms)

@@ -341,12 +341,18 @@ __global__ __launch_bounds__(64) void exp_gates_kernel(const float* __restrict__
             i = cap * tanhf((gi[(size_t)t * ldg + h] + b_i) * inv_cap);
             f = log_sigmoid_f32(cap * tanhf((gf[(size_t)t * ldg + h] + b_f) * inv_cap));
         }
+        // (lane j's gates by a read of that lane with j known at compile time: the walk's chain is then an addition and a
+        // maximum a token, and the 128 reads do not stand in it)
         float before = 0.0f, mine = 0.0f;
-        for (int j = 0; j < n_here; ++j) {
-            float fj = __shfl(f, j, 64), ij = __shfl(i, j, 64);
-            float m_new = fmaxf(fj + m, ij);
-            if (lane == j) { before = m; mine = m_new; }
-            m = m_new;
+#pragma unroll
+        for (int j = 0; j < 64; ++j) {
+            if (j < n_here) {
+                float fj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(f), j));
+                float ij = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(i), j));
+                float m_new = fmaxf(fj + m, ij);
+                if (lane == j) { before = m; mine = m_new; }
+                m = m_new;
+            }
         }
         if (in) {
             decay[(size_t)t * ldo + h] = expf(f + before - mine);

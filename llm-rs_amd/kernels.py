@@ -20,7 +20,9 @@ from typing import Dict, List, NamedTuple, Optional
 import torch
 
 EPI_STORE, EPI_STORE_F32, EPI_ACCUM_F32, EPI_SWIGLU = 0, 1, 2, 3
-_EPI_NAMES = {EPI_STORE: "store", EPI_STORE_F32: "store32", EPI_ACCUM_F32: "add32", EPI_SWIGLU: "swiglu"}
+EPI_GLU_CLAMP = 5       # (4 is the kernel library's own: the q/k/v epilogue of `qkv_rope_cache`)
+_EPI_NAMES = {EPI_STORE: "store", EPI_STORE_F32: "store32", EPI_ACCUM_F32: "add32", EPI_SWIGLU: "swiglu", EPI_GLU_CLAMP: "clamped glu"}
+_EPI_GATED = (EPI_SWIGLU, EPI_GLU_CLAMP)
 
 _DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
 
@@ -187,7 +189,7 @@ class HipKernels(Kernels):
             "llmrs_cast": [V, V, I, V, I, c_size_t],
             "llmrs_scale_softcap_rows": [V, V, I, I, I, F, F],
             "llmrs_rmsnorm": [V, I, V, V, V, V, I, I, F],
-            "llmrs_gemm": [V, I, V, I, V, V, I, I, I, I, I, V, c_size_t, I, V, I, F, V, V, I, V, F],
+            "llmrs_gemm": [V, I, V, I, V, V, I, I, I, I, I, V, c_size_t, I, V, I, F, V, V, I, V, F, F, F],
             "llmrs_gemm_defers_norm": [I, I, I],
             "llmrs_gemm_norms_whole": [I, I, I],
             "llmrs_gemm_next_parts": [I, I, I],
@@ -431,8 +433,11 @@ class HipKernels(Kernels):
 
     # out (epilogue) a @ w.T ; a: [M, K] rows may be strided, w: [N, K] dense
     def gemm(self, a, w: torch.Tensor, out: torch.Tensor, epilogue: int = EPI_STORE,
-             workspace: Optional[torch.Tensor] = None, leave: Optional[NextNorm] = None) -> None:
-        """`a` may be `NormedRows`, and `leave` a `NextNorm` (with the += epilogue), where `gemm_defers_norm` holds."""
+             workspace: Optional[torch.Tensor] = None, leave: Optional[NextNorm] = None, glu=None) -> None:
+        """`a` may be `NormedRows`, and `leave` a `NextNorm` (with the += epilogue), where `gemm_defers_norm` holds.
+        EPI_GLU_CLAMP (rows of w are gate_0, up_0, gate_1, ...; glu = (limit, alpha)): out[m, j] = g sigmoid(alpha g) (u + 1)
+        with g = min(gate_j, limit), u = clamp(up_j, -limit, limit), computed on the 32-bit sums, in the activation type."""
+        assert (glu is not None) == (epilogue == EPI_GLU_CLAMP)
         scale = None
         if isinstance(a, NormedRows):
             scale, a = a, a.y
@@ -452,7 +457,7 @@ class HipKernels(Kernels):
         elif scale is not None or leave is not None:
             assert a.dtype == torch.bfloat16 and self.gemm_defers_norm(M, N, K)
         want = torch.float32 if epilogue in (EPI_STORE_F32, EPI_ACCUM_F32) else a.dtype
-        assert out.dtype == want and out.shape[0] == M and out.shape[1] == (N // 2 if epilogue == EPI_SWIGLU else N)
+        assert out.dtype == want and out.shape[0] == M and out.shape[1] == (N // 2 if epilogue in _EPI_GATED else N)
         moved = (M * K + N * K) * a.element_size() + out.numel() * out.element_size() * (2 if epilogue == EPI_ACCUM_F32 else 1)
         label = f"gemm {M}x{N}x{K} {'norm+' if scale is not None else ''}{_EPI_NAMES[epilogue]}{('+norm' if whole else '+next') if leave is not None else ''}"
         self._run(label, moved, 2 * M * N * K, a.dtype,
@@ -462,7 +467,8 @@ class HipKernels(Kernels):
                   None if scale is None else _p(scale.sumsq), 0 if scale is None else scale.sumsq.shape[1],
                   0.0 if scale is None else scale.eps, None if leave is None or whole else _p(leave.sumsq),
                   None if leave is None else _p(leave.y), 0 if leave is None else leave.y.stride(0),
-                  None if leave is None else _p(leave.weight), leave.eps if whole else 0.0)
+                  None if leave is None else _p(leave.weight), leave.eps if whole else 0.0,
+                  0.0 if glu is None else float(glu[0]), 0.0 if glu is None else float(glu[1]))
 
     def rope_kv_write(self, qkv, positions, slot_map, inv_freq, rotary_dim, interleaved, k_cache, v_cache,
                       n_heads, n_kv_heads, head_dim, page_size, num_pages, write_kv) -> None:

@@ -8,7 +8,7 @@ from __future__ import annotations
 
 import torch
 
-from ..kernels import EPI_ACCUM_F32, EPI_STORE_F32, EPI_SWIGLU, kernels
+from ..kernels import EPI_ACCUM_F32, EPI_GLU_CLAMP, EPI_STORE_F32, EPI_SWIGLU, kernels
 from .base import FeedForward, TensorSpec, build_feed_forward, place, register_feed_forward
 
 
@@ -63,8 +63,9 @@ GATED = ("clamped_glu",)                     # activations of two projections, g
 class ClampedGLU(FeedForward):
     """Feed-forward with a clamped, gated activation(hidden_size, intermediate_size, limit, alpha):
     h += Wdown (g sigmoid(alpha g) (u + 1)), g = min(Wgate x, limit), u = clamp(Wup x, -limit, limit); alpha is 1.702
-    unless given.  The gate and up weights are interleaved row by row at load, so one product leaves (gate_j, up_j) side
-    by side as 32-bit sums; the activation is computed on them and rounded once to the activation type."""
+    unless given.  The gate and up weights are interleaved row by row at load, so one product yields (gate_j, up_j) side
+    by side and its epilogue writes the activation, computed on the 32-bit sums and rounded once; the down product adds
+    into the 32-bit stream."""
     graph_safe = True
 
     def __init__(self, spec, dtype):
@@ -94,10 +95,8 @@ class ClampedGLU(FeedForward):
     def forward(self, ctx, x, h):
         k = kernels()
         T = x.shape[0]
-        sums = ctx.workspace("mlp.up", (T, 2 * self.inter), torch.float32)
-        k.gemm(x, self.w_gate_up, sums, EPI_STORE_F32, ctx.gemm_workspace(x, self.w_gate_up))
         act = ctx.workspace("mlp.act", (T, self.inter), self.dtype)
-        k.act_weight(act, sums, None, self.inter, "clamped_glu", self.limit, self.alpha)
+        k.gemm(x, self.w_gate_up, act, EPI_GLU_CLAMP, ctx.gemm_workspace(x, self.w_gate_up), glu=(self.limit, self.alpha))
         k.gemm(act, self.w_down, h, EPI_ACCUM_F32, ctx.gemm_workspace(act, self.w_down))
         ctx.note_left(h, None)
 

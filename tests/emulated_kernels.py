@@ -11,7 +11,7 @@ import torch
 
 from llm_rs_amd.kernels import Kernels, NormPlan
 
-EPI_STORE, EPI_STORE_F32, EPI_ACCUM_F32, EPI_SWIGLU = 0, 1, 2, 3
+EPI_STORE, EPI_STORE_F32, EPI_ACCUM_F32, EPI_SWIGLU, EPI_GLU_CLAMP = 0, 1, 2, 3, 5
 
 
 class EmulatedKernels(Kernels):
@@ -119,7 +119,7 @@ class EmulatedKernels(Kernels):
     def norm_left_by_product(self, M, N, K, dtype):
         return NormPlan(False, -(-N // 16)) if dtype == torch.bfloat16 and 1 <= M <= 16 else None
 
-    def gemm(self, a, w, out, epilogue=EPI_STORE, workspace=None, leave=None):
+    def gemm(self, a, w, out, epilogue=EPI_STORE, workspace=None, leave=None, glu=None):
         inv = None
         if hasattr(a, "sumsq"):        # kernels.NormedRows: rows times the norm's weight, rounded; the scale comes after the sums
             inv = 1.0 / torch.sqrt(a.sumsq.sum(-1, keepdim=True) / a.y.shape[1] + a.eps)
@@ -139,6 +139,10 @@ class EmulatedKernels(Kernels):
             out.copy_(acc)
         elif epilogue == EPI_ACCUM_F32:
             out.add_(acc)
+        elif epilogue == EPI_GLU_CLAMP:
+            limit, alpha = glu
+            g, u = torch.clamp(acc[:, 0::2], max=limit), torch.clamp(acc[:, 1::2], min=-limit, max=limit)
+            out.copy_((g * torch.sigmoid(alpha * g) * (u + 1.0)).to(out.dtype))
         else:
             g, u = acc[:, 0::2], acc[:, 1::2]
             out.copy_((g / (1.0 + torch.exp(-g)) * u).to(out.dtype))

@@ -147,6 +147,26 @@ def test_the_router_with_sigmoid_scores_and_a_correction(E, top):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("M", [1, 2, 8, 16, 17, 40, 64, 65, 100, 300, 1031, 2048])
+@pytest.mark.parametrize("N,K", [(14, 10), (64, 64), (512, 320), (2048, 256), (6144, 1024)])
+def test_the_gate_and_up_product_with_the_clamped_activation(M, N, K, dtype):
+    """Every tiling of the product (by its number of rows and its widths) finishes the same activation; two different
+    limits one after the other, as two feed-forwards of a layer have them."""
+    from llm_rs_amd.kernels import EPI_GLU_CLAMP
+    x, w = (rand(M, K, seed=M) * 0.8).to(dtype), (rand(N, K, seed=N) * 0.2).to(dtype)
+    sums = x.double() @ w.double().T
+    for limit, alpha in ((1.25, 1.702), (0.5, 1.0)):
+        g, u = torch.clamp(sums[:, 0::2], max=limit), torch.clamp(sums[:, 1::2], min=-limit, max=limit)
+        want = g * plain_sigmoid(alpha * g) * (u + 1.0)
+        out = torch.empty(M, N // 2, dtype=dtype, device="cuda")
+        k = kernels()
+        n_ws = k.gemm_workspace_floats(M, N, K)
+        ws = torch.empty(n_ws, device="cuda") if n_ws else None
+        k.gemm(x.cuda(), w.cuda(), out, EPI_GLU_CLAMP, ws, glu=(limit, alpha))
+        close(out, want, dtype, f"limit {limit}", tol=5e-5 if dtype == torch.float32 else 1e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_the_clamped_gated_activation(dtype):
     T, ff, E = 19, 6, 3
     sums = rand(T, 2 * ff * E, seed=3) * 3.0
