@@ -333,13 +333,22 @@ __global__ __launch_bounds__(64) void exp_gates_kernel(const float* __restrict__
     float* mp = m_state + (size_t)slots[e] * state_stride + h;
     float m = *mp;
     const float b_i = bi ? bi[h] : 0.0f, b_f = bf ? bf[h] : 0.0f, inv_cap = 1.0f / cap;
+    // (a chunk's raw gates are asked for a chunk ahead: a lane reads a row of its own, a trip to memory that the walk
+    // of the chunk before hides)
+    float raw_i = t0 + lane < t1 ? gi[(size_t)(t0 + lane) * ldg + h] : 0.0f;
+    float raw_f = t0 + lane < t1 ? gf[(size_t)(t0 + lane) * ldg + h] : 0.0f;
     for (int tc = t0; tc < t1; tc += 64) {
         const int t = tc + lane, n_here = min(64, t1 - tc);
         const bool in = t < t1;
+        const float now_i = raw_i, now_f = raw_f;
+        if (t + 64 < t1) {
+            raw_i = gi[(size_t)(t + 64) * ldg + h];
+            raw_f = gf[(size_t)(t + 64) * ldg + h];
+        }
         float i = 0.0f, f = 0.0f;
         if (in) {
-            i = cap * tanhf((gi[(size_t)t * ldg + h] + b_i) * inv_cap);
-            f = log_sigmoid_f32(cap * tanhf((gf[(size_t)t * ldg + h] + b_f) * inv_cap));
+            i = cap * tanhf((now_i + b_i) * inv_cap);
+            f = log_sigmoid_f32(cap * tanhf((now_f + b_f) * inv_cap));
         }
         // (lane j's gates by a read of that lane with j known at compile time: the walk's chain is then an addition and a
         // maximum a token, and the 128 reads do not stand in it)
