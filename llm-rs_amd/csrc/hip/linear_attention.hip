@@ -317,59 +317,66 @@ extern "C" int llmrs_delta_prepare(hipStream_t stream, float* q, int ldq, float*
 //   f = log sigmoid(cap tanh((gf + bf) / cap))     the forget gate's logarithm
 //   m_t = max(f + m_(t-1), i)                      the running maximum, carried in the request's state (it starts at 0)
 //   decay = exp(f + m_(t-1) - m_t),  take = exp(i - m_t),  floor = exp(-m_t)
-// One wave for each (entry, head): the gates of 64 tokens at a time, a token a lane; the maximum walks over them in
-// order, one addition and one comparison a token, exactly as token-by-token steps would, so a prompt cut anywhere gives
-// the same bits.
+// One block of four waves for each (entry, head), 256 tokens a round, a token a thread: the gates' logarithms (two tanh,
+// a log sigmoid) side by side in all four waves; then the first wave walks the maximum over the round's tokens in order,
+// one addition and one comparison a token, exactly as token-by-token steps would, so a prompt cut anywhere gives the
+// same bits; then all four waves finish their tokens' three exponentials.
 __device__ __forceinline__ float log_sigmoid_f32(float z) { return z >= 0.0f ? -log1pf(expf(-z)) : z - log1pf(expf(z)); }
 
-__global__ __launch_bounds__(64) void exp_gates_kernel(const float* __restrict__ gi, const float* __restrict__ gf, int ldg,
-                                                        const float* __restrict__ bi, const float* __restrict__ bf, float cap,
-                                                        float* __restrict__ m_state, long state_stride, const int* __restrict__ q_starts,
-                                                        const int* __restrict__ slots, float* __restrict__ decay,
-                                                        float* __restrict__ take, float* __restrict__ floor_, int ldo) {
-    const int h = blockIdx.x, e = blockIdx.y, lane = threadIdx.x;
+#define GATES_THREADS 256
+__global__ __launch_bounds__(GATES_THREADS) void exp_gates_kernel(const float* __restrict__ gi, const float* __restrict__ gf, int ldg,
+                                                                   const float* __restrict__ bi, const float* __restrict__ bf, float cap,
+                                                                   float* __restrict__ m_state, long state_stride,
+                                                                   const int* __restrict__ q_starts, const int* __restrict__ slots,
+                                                                   float* __restrict__ decay, float* __restrict__ take,
+                                                                   float* __restrict__ floor_, int ldo) {
+    __shared__ float si[GATES_THREADS], sf[GATES_THREADS], s_before[GATES_THREADS], s_mine[GATES_THREADS];
+    const int h = blockIdx.x, e = blockIdx.y, tid = threadIdx.x, lane = tid & 63;
     const int t0 = q_starts[e], t1 = q_starts[e + 1];
     if (t0 >= t1) return;
     float* mp = m_state + (size_t)slots[e] * state_stride + h;
-    float m = *mp;
+    float m = *mp;                          // (every thread carries it; only the first wave's is kept up to date)
     const float b_i = bi ? bi[h] : 0.0f, b_f = bf ? bf[h] : 0.0f, inv_cap = 1.0f / cap;
-    // (a chunk's raw gates are asked for a chunk ahead: a lane reads a row of its own, a trip to memory that the walk
-    // of the chunk before hides)
-    float raw_i = t0 + lane < t1 ? gi[(size_t)(t0 + lane) * ldg + h] : 0.0f;
-    float raw_f = t0 + lane < t1 ? gf[(size_t)(t0 + lane) * ldg + h] : 0.0f;
-    for (int tc = t0; tc < t1; tc += 64) {
-        const int t = tc + lane, n_here = min(64, t1 - tc);
+    for (int tc = t0; tc < t1; tc += GATES_THREADS) {
+        const int t = tc + tid, n_here = min(GATES_THREADS, t1 - tc);
         const bool in = t < t1;
-        const float now_i = raw_i, now_f = raw_f;
-        if (t + 64 < t1) {
-            raw_i = gi[(size_t)(t + 64) * ldg + h];
-            raw_f = gf[(size_t)(t + 64) * ldg + h];
-        }
-        float i = 0.0f, f = 0.0f;
+        // (a place past the entry's end holds gates that leave the maximum as it is, bit for bit: m + 0 against minus
+        // infinity; the walk then needs no count)
+        float i = -INFINITY, f = 0.0f;
         if (in) {
-            i = cap * tanhf((now_i + b_i) * inv_cap);
-            f = log_sigmoid_f32(cap * tanhf((now_f + b_f) * inv_cap));
+            i = cap * tanhf((gi[(size_t)t * ldg + h] + b_i) * inv_cap);
+            f = log_sigmoid_f32(cap * tanhf((gf[(size_t)t * ldg + h] + b_f) * inv_cap));
         }
-        // (lane j's gates by a read of that lane with j known at compile time: the walk's chain is then an addition and a
-        // maximum a token, and the 128 reads do not stand in it)
-        float before = 0.0f, mine = 0.0f;
+        si[tid] = i;
+        sf[tid] = f;
+        __syncthreads();
+        if (tid < 64) {
+            for (int sub = 0; sub < n_here; sub += 64) {
+                const float fi = si[sub + lane], ff = sf[sub + lane];
+                // (lane j's gates by a read of that lane with j known at compile time: the walk's chain is then an
+                // addition and a maximum a token, and the 128 reads do not stand in it)
+                float before = 0.0f, mine = 0.0f;
 #pragma unroll
-        for (int j = 0; j < 64; ++j) {
-            if (j < n_here) {
-                float fj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(f), j));
-                float ij = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(i), j));
-                float m_new = fmaxf(fj + m, ij);
-                if (lane == j) { before = m; mine = m_new; }
-                m = m_new;
+                for (int j = 0; j < 64; ++j) {
+                    float fj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(ff), j));
+                    float ij = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(fi), j));
+                    float m_new = fmaxf(fj + m, ij);
+                    if (lane == j) { before = m; mine = m_new; }
+                    m = m_new;
+                }
+                s_before[sub + lane] = before;
+                s_mine[sub + lane] = mine;
             }
         }
+        __syncthreads();
         if (in) {
+            const float before = s_before[tid], mine = s_mine[tid];
             decay[(size_t)t * ldo + h] = expf(f + before - mine);
             take[(size_t)t * ldo + h] = expf(i - mine);
             floor_[(size_t)t * ldo + h] = expf(-mine);
         }
     }
-    if (lane == 0) *mp = m;
+    if (tid == 0) *mp = m;
 }
 
 // gi, gf: [T, ldg] 32-bit, head h's raw gate at column h; bi, bf: [heads] or null; m_state: a request's maxima at
@@ -381,7 +388,7 @@ extern "C" int llmrs_exp_gates(hipStream_t stream, const float* gi, const float*
     LLMRS_REQUIRE(cap > 0.0f, "exp_gates: the gates' cap must be positive, got %g", cap);
     LLMRS_REQUIRE(q_starts && slots && n_entries > 0 && n_entries <= 65535, "exp_gates: bad entries");
     if (n_tokens == 0) return 0;
-    exp_gates_kernel<<<dim3(heads, n_entries), 64, 0, stream>>>(gi, gf, ldg, bi, bf, cap, m_state, state_stride, q_starts, slots, decay, take, floor_, ldo);
+    exp_gates_kernel<<<dim3(heads, n_entries), GATES_THREADS, 0, stream>>>(gi, gf, ldg, bi, bf, cap, m_state, state_stride, q_starts, slots, decay, take, floor_, ldo);
     LLMRS_LAUNCH_CHECK("exp_gates");
     return 0;
 }
