@@ -11,28 +11,32 @@ enum LlmrsEpilogue {
                               // out[m, n/2] = silu(acc[m, n]) * acc[m, n+1] for even n, activation type
     LLMRS_EPI_QKV = 4,        // rows of W are q heads, k heads, v heads: rotate q and k (adjacent pairs),
                               // q to out, k and v straight into the paged cache (QkvEpilogue)
-    LLMRS_EPI_GLU_CLAMP = 5,  // rows of W as for SWIGLU: with g = min(acc[m, n], limit), u = clamp(acc[m, n+1], -limit, limit),
-                              // out[m, n/2] = g * sigmoid(alpha * g) * (u + 1), activation type (GluClamp)
+    LLMRS_EPI_GLU_CLAMP = 5,  // 5 + slot, slot < LLMRS_GLU_SLOTS: rows of W as for SWIGLU; with the slot's constants (GluClamp),
+                              // g = min(acc[m, n], limit), u = clamp(acc[m, n+1], -limit, limit),
+                              // out[m, n/2] = g * sigmoid(alpha * g) * (u + 1), activation type
 };
 
-// The constants of the clamped gated epilogue.  A kernel finds them in device memory (a variable of its own source
-// file), where a one-thread kernel launched right before it on the same stream has put them: kernels of one stream
-// run in order, also as nodes of a recorded graph, and nothing else of a product's launch changes.
+// The constants of the clamped gated epilogue lie in a table in device memory, a slot for each pair of them that a
+// model has (llmrs_glu_clamp_slot, called when a feed-forward takes its weights, writes a slot once and for all); the
+// epilogue's number says which slot, so no kernel's argument list holds them and a recorded step finds them as any
+// other does.  Each source file with such kernels has the table for itself (the variable is static).
+#define LLMRS_GLU_SLOTS 64
 struct GluClamp {
     float limit, alpha;
 };
-static __device__ GluClamp llmrs_glu_clamp;
-static __global__ void glu_clamp_set_kernel(GluClamp p) { llmrs_glu_clamp = p; }
-static inline void glu_clamp_set(hipStream_t stream, const GluClamp& p) { glu_clamp_set_kernel<<<1, 1, 0, stream>>>(p); }
+static __device__ GluClamp llmrs_glu_clamp[LLMRS_GLU_SLOTS];
+static __global__ void glu_clamp_store_kernel(int slot, GluClamp p) { llmrs_glu_clamp[slot] = p; }
+// (gemm_mfma.hip: the same slot of that file's table)
+void llmrs_glu_clamp_store_mfma(hipStream_t stream, int slot, GluClamp p);
 
-__host__ __device__ __forceinline__ bool epi_gated(int epi) { return epi == LLMRS_EPI_SWIGLU || epi == LLMRS_EPI_GLU_CLAMP; }
-// act(gate, up) of the two gated epilogues, on 32-bit sums
+__host__ __device__ __forceinline__ bool epi_gated(int epi) { return epi == LLMRS_EPI_SWIGLU || epi >= LLMRS_EPI_GLU_CLAMP; }
+// act(gate, up) of the gated epilogues, on 32-bit sums
 __device__ __forceinline__ float gated_act(int epi, float g, float u) {
     if (epi == LLMRS_EPI_SWIGLU) return silu_f32(g) * u;
-    const float limit = llmrs_glu_clamp.limit;
-    g = fminf(g, limit);
-    u = fminf(fmaxf(u, -limit), limit);
-    return g / (1.0f + expf(-llmrs_glu_clamp.alpha * g)) * (u + 1.0f);
+    const GluClamp p = llmrs_glu_clamp[epi - LLMRS_EPI_GLU_CLAMP];
+    g = fminf(g, p.limit);
+    u = fminf(fmaxf(u, -p.limit), p.limit);
+    return g / (1.0f + expf(-p.alpha * g)) * (u + 1.0f);
 }
 
 // What the q/k/v epilogue needs beside the sums.
@@ -89,11 +93,9 @@ __device__ __forceinline__ void epilogue_store(int epi, void* out, int ldc, int 
 // parts, 0 when this product would not be split (nothing launched), -1 on error.
 int llmrs_gemm_bf16_split_parts(hipStream_t stream, const bf16* A, int lda, const bf16* W, int M, int N, int K,
                                 void* workspace, size_t workspace_bytes);
-// glu: the constants of LLMRS_EPI_GLU_CLAMP (put into this source file's device variable before any kernel is launched).
 int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16* W, void* out, int ldc,
                          int M, int N, int K, int epi, void* workspace, size_t workspace_bytes,
-                         const QkvEpilogue* qkv = nullptr, const RowScale* scale = nullptr, const NextNorm* next = nullptr,
-                         const GluClamp* glu = nullptr);
+                         const QkvEpilogue* qkv = nullptr, const RowScale* scale = nullptr, const NextNorm* next = nullptr);
 // Whether the bfloat16 product of this shape goes to the kernel that can scale its rows' sums and leave a NextNorm.
 extern "C" int llmrs_gemm_defers_norm(int M, int N, int K);
 // The parts per row of the sums of squares that such a product leaves (NextNorm): what the caller sizes sumsq by.

@@ -56,11 +56,12 @@ __device__ __forceinline__ float silu_fast_f32(float x) {
 // act(gate, up) of the two gated epilogues with the same instructions
 __device__ __forceinline__ float gated_act_fast(int epi, float g, float u) {
     if (epi == LLMRS_EPI_SWIGLU) return silu_fast_f32(g) * u;
-    const float limit = llmrs_glu_clamp.limit;
-    g = fminf(g, limit);
-    u = fminf(fmaxf(u, -limit), limit);
-    return g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g * (llmrs_glu_clamp.alpha * -1.44269504088896341f))) * (u + 1.0f);
+    const GluClamp p = llmrs_glu_clamp[epi - LLMRS_EPI_GLU_CLAMP];
+    g = fminf(g, p.limit);
+    u = fminf(fmaxf(u, -p.limit), p.limit);
+    return g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g * (p.alpha * -1.44269504088896341f))) * (u + 1.0f);
 }
+void llmrs_glu_clamp_store_mfma(hipStream_t stream, int slot, GluClamp p) { glu_clamp_store_kernel<<<1, 1, 0, stream>>>(slot, p); }
 
 // The tile loops' barrier: this wave's LDS reads and writes are done, then every wave of the block
 // has arrived.  Unlike __syncthreads() it does not wait for loads from memory that are still in
@@ -1007,9 +1008,10 @@ static int launch_pingpong(hipStream_t stream, const bf16* A, int lda, const bf1
 // What a wave of the four-wave tile does with its sums: one band of 32 rows at a time.  16-bit results go through
 // the wave's own part of LDS and leave as whole rows of the band, 16 bytes a lane; the 32-bit epilogues read and
 // write memory directly (a lane half holds 32 consecutive columns of a row: whole lines).
+// epi: the epilogue's number as the caller gave it (EPI with its slot, where it has one)
 template <int BM, int BN, int EPI>
 __device__ __forceinline__ void band_epilogue(f32x16 (&acc)[BM / 64][BN / 64], unsigned char* smem, void* __restrict__ out,
-                                              int ldc, int M, int N, int m0, int n0) {
+                                              int ldc, int M, int N, int m0, int n0, int epi) {
     constexpr int TM = BM / 2, TN = BN / 2, FM = TM / 32, FN = TN / 32;
     int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     int wm = wave / 2, wn = wave % 2;
@@ -1051,7 +1053,7 @@ __device__ __forceinline__ void band_epilogue(f32x16 (&acc)[BM / 64][BN / 64], u
                     float v0 = acc[i][j][r], v1 = acc[i][j][r + 1];
                     float got = swap_neighbours(odd ? v0 : v1);
                     float left = odd ? got : v0, right = odd ? v1 : got;
-                    if (glu) *(bf16*)(mine + row * row_bytes + (cc / 2) * 2) = (bf16)gated_act_fast(EPI, left, right);
+                    if (glu) *(bf16*)(mine + row * row_bytes + (cc / 2) * 2) = (bf16)gated_act_fast(EPI == LLMRS_EPI_GLU_CLAMP ? epi : EPI, left, right);
                     else {
                         bf16x2 two;
                         two[0] = (bf16)left;
@@ -1077,7 +1079,7 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 template <int BM, int BN, int EPI>
 __global__ __launch_bounds__(256) void gemm_fourwave_kernel(const bf16* __restrict__ A, int lda, const bf16* __restrict__ W,
-                                                            void* __restrict__ out, int ldc, int M, int N, int K) {
+                                                            void* __restrict__ out, int ldc, int M, int N, int K, int epi) {
     extern __shared__ __attribute__((aligned(1024))) unsigned char fw_smem[];
     constexpr int WAVES = 4;
     constexpr int TM = BM / 2, TN = BN / 2, FM = TM / 32, FN = TN / 32;
@@ -1211,7 +1213,7 @@ __global__ __launch_bounds__(256) void gemm_fourwave_kernel(const bf16* __restri
     mult(I1{});
     wait_vmcnt<0>();
     __syncthreads();
-    band_epilogue<BM, BN, EPI>(acc, fw_smem, out, ldc, M, N, m0, n0);
+    band_epilogue<BM, BN, EPI>(acc, fw_smem, out, ldc, M, N, m0, n0, epi);
 }
 
 // Whether the four-wave tiles can finish this product: the epilogues it has, 16-bit results as whole 16-byte pieces.
@@ -1222,7 +1224,7 @@ static bool fourwave_takes(int epi, const void* out, int ldc, int N) {
     return false;
 }
 template <int BM, int BN, int EPI>
-static int launch_fourwave_epi(hipStream_t stream, const bf16* A, int lda, const bf16* W, void* out, int ldc, int M, int N, int K) {
+static int launch_fourwave_epi(hipStream_t stream, const bf16* A, int lda, const bf16* W, void* out, int ldc, int M, int N, int K, int epi) {
     static bool configured = false;
     size_t bytes = (size_t)2 * (BM + BN) * 128;
     if (!configured) {
@@ -1233,18 +1235,18 @@ static int launch_fourwave_epi(hipStream_t stream, const bf16* A, int lda, const
     }
     dim3 grid(ceil_div(N, BN), ceil_div(M, BM));
     if (grid.y > 65535) return llmrs_fail("gemm: M=%d is too large for one launch", M);
-    gemm_fourwave_kernel<BM, BN, EPI><<<grid, 256, bytes, stream>>>(A, lda, W, out, ldc, M, N, K);
+    gemm_fourwave_kernel<BM, BN, EPI><<<grid, 256, bytes, stream>>>(A, lda, W, out, ldc, M, N, K, epi);
     return 0;
 }
 // (operands under 4 GB each, K % 64 == 0, fourwave_takes(epi, ...): the caller's to check)
 template <int BM, int BN>
 static int launch_fourwave(hipStream_t stream, const bf16* A, int lda, const bf16* W, void* out, int ldc, int M, int N, int K, int epi) {
+    if (epi >= LLMRS_EPI_GLU_CLAMP) return launch_fourwave_epi<BM, BN, LLMRS_EPI_GLU_CLAMP>(stream, A, lda, W, out, ldc, M, N, K, epi);
     switch (epi) {
-        case LLMRS_EPI_STORE: return launch_fourwave_epi<BM, BN, LLMRS_EPI_STORE>(stream, A, lda, W, out, ldc, M, N, K);
-        case LLMRS_EPI_STORE_F32: return launch_fourwave_epi<BM, BN, LLMRS_EPI_STORE_F32>(stream, A, lda, W, out, ldc, M, N, K);
-        case LLMRS_EPI_ACCUM_F32: return launch_fourwave_epi<BM, BN, LLMRS_EPI_ACCUM_F32>(stream, A, lda, W, out, ldc, M, N, K);
-        case LLMRS_EPI_SWIGLU: return launch_fourwave_epi<BM, BN, LLMRS_EPI_SWIGLU>(stream, A, lda, W, out, ldc, M, N, K);
-        case LLMRS_EPI_GLU_CLAMP: return launch_fourwave_epi<BM, BN, LLMRS_EPI_GLU_CLAMP>(stream, A, lda, W, out, ldc, M, N, K);
+        case LLMRS_EPI_STORE: return launch_fourwave_epi<BM, BN, LLMRS_EPI_STORE>(stream, A, lda, W, out, ldc, M, N, K, epi);
+        case LLMRS_EPI_STORE_F32: return launch_fourwave_epi<BM, BN, LLMRS_EPI_STORE_F32>(stream, A, lda, W, out, ldc, M, N, K, epi);
+        case LLMRS_EPI_ACCUM_F32: return launch_fourwave_epi<BM, BN, LLMRS_EPI_ACCUM_F32>(stream, A, lda, W, out, ldc, M, N, K, epi);
+        case LLMRS_EPI_SWIGLU: return launch_fourwave_epi<BM, BN, LLMRS_EPI_SWIGLU>(stream, A, lda, W, out, ldc, M, N, K, epi);
         default: return llmrs_fail("gemm: the four-wave tiles have no epilogue %d", epi);
     }
 }
@@ -1363,12 +1365,11 @@ int llmrs_gemm_bf16_split_parts(hipStream_t stream, const bf16* A, int lda, cons
 
 int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16* W, void* out, int ldc,
                          int M, int N, int K, int epi, void* workspace, size_t workspace_bytes,
-                         const QkvEpilogue* qkv, const RowScale* scale, const NextNorm* next, const GluClamp* glu) {
+                         const QkvEpilogue* qkv, const RowScale* scale, const NextNorm* next) {
     if (K % 8 || lda % 8 || ((uintptr_t)A & 15) || ((uintptr_t)W & 15)) {
         if (scale != nullptr || next != nullptr) { llmrs_fail("gemm: a deferred norm needs rows of a multiple of 8 values, 16-byte aligned"); return -1; }
         return 0;
     }
-    if (glu != nullptr) glu_clamp_set(stream, *glu);      // (a call that hands part of its rows on to itself has set them already)
     const bool whole = next != nullptr && next->eps > 0.0f;      // the norm that follows is finished by the kernel that adds the parts up
     if (whole) {
         bool ok = scale == nullptr && epi == LLMRS_EPI_ACCUM_F32 && llmrs_gemm_norms_whole(M, N, K) && workspace != nullptr &&

@@ -336,6 +336,38 @@ static void launch_f32_skinny(hipStream_t stream, const float* A, int lda, const
     gemm_f32_skinny_kernel<NT, NW, U><<<ceil_div(N, NT * 16), NW * 64, bytes, stream>>>(A, lda, W, out, ldc, M, N, K, epi);
 }
 
+// ---- the slots of the clamped gated epilogue's constants -------------------------------------------------------------
+// A pair (limit, alpha) gets a slot the first time a feed-forward asks for it on a device (when it takes its weights:
+// never inside a recording); the slot is written in both source files' tables and the stream is waited for, so every
+// later product on any stream finds it.  The same pair on the same device gets the same slot again.
+#include <mutex>
+#include <vector>
+struct GluSlot { int device; float limit, alpha; };
+static std::mutex glu_mutex;
+static std::vector<GluSlot> glu_slots;
+static int glu_clamp_slots_taken() {
+    std::lock_guard<std::mutex> lock(glu_mutex);
+    return (int)glu_slots.size();
+}
+extern "C" int llmrs_glu_clamp_slot(hipStream_t stream, float limit, float alpha) {
+    if (!(limit > 0.0f)) { llmrs_fail("glu_clamp_slot: the limit must be positive, got %g", limit); return -1; }
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess) { llmrs_fail("glu_clamp_slot: no current device"); return -1; }
+    std::lock_guard<std::mutex> lock(glu_mutex);
+    for (size_t i = 0; i < glu_slots.size(); ++i)
+        if (glu_slots[i].device == device && glu_slots[i].limit == limit && glu_slots[i].alpha == alpha) return (int)i;
+    if (glu_slots.size() >= LLMRS_GLU_SLOTS) { llmrs_fail("glu_clamp_slot: more than %d different pairs of constants", LLMRS_GLU_SLOTS); return -1; }
+    int slot = (int)glu_slots.size();
+    GluClamp p{limit, alpha};
+    glu_clamp_store_kernel<<<1, 1, 0, stream>>>(slot, p);
+    llmrs_glu_clamp_store_mfma(stream, slot, p);
+    hipError_t e = hipGetLastError();
+    if (e == hipSuccess) e = hipStreamSynchronize(stream);
+    if (e != hipSuccess) { llmrs_fail("glu_clamp_slot: %s", hipGetErrorString(e)); return -1; }
+    glu_slots.push_back(GluSlot{device, limit, alpha});
+    return slot;
+}
+
 // A: [M, K] with row stride lda; W: [N, K] dense; out: row stride ldc (elements of
 // its own type; for SWIGLU the output has N/2 columns).  workspace: optional device
 // memory (16 * 64 * N * 4 bytes is always enough) for products that split K over blocks.
@@ -346,12 +378,11 @@ static void launch_f32_skinny(hipStream_t stream, const float* A, int lda, const
 extern "C" int llmrs_gemm(hipStream_t stream, int dtype, const void* A, int lda, const void* W, void* out, int ldc,
                           int M, int N, int K, int epi, void* workspace, size_t workspace_bytes, int allow_mfma,
                           const float* scale_sumsq, int scale_parts, float scale_eps, float* next_sumsq, void* next_y,
-                          int next_ldy, const float* next_weight, float next_eps, float glu_limit, float glu_alpha) {
+                          int next_ldy, const float* next_weight, float next_eps) {
     LLMRS_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
     LLMRS_REQUIRE(lda >= K, "gemm: row stride %d of A is shorter than K=%d", lda, K);
-    LLMRS_REQUIRE((epi >= 0 && epi <= 3) || epi == LLMRS_EPI_GLU_CLAMP, "gemm: unknown epilogue %d", epi);
-    LLMRS_REQUIRE(epi != LLMRS_EPI_GLU_CLAMP || glu_limit > 0.0f, "gemm: the clamped gated epilogue needs a positive limit, got %g", glu_limit);
-    const GluClamp glu{glu_limit, glu_alpha};
+    LLMRS_REQUIRE((epi >= 0 && epi <= 3) || (epi >= LLMRS_EPI_GLU_CLAMP && epi < LLMRS_EPI_GLU_CLAMP + glu_clamp_slots_taken()),
+                  "gemm: unknown epilogue %d (a clamped gated epilogue is %d + a slot that llmrs_glu_clamp_slot gave)", epi, (int)LLMRS_EPI_GLU_CLAMP);
     if (epi_gated(epi)) {
         LLMRS_REQUIRE(N % 2 == 0, "gemm: the gate/up epilogue needs an even N, got %d", N);
         LLMRS_REQUIRE(ldc >= N / 2, "gemm: row stride %d of out is shorter than N/2=%d", ldc, N / 2);
@@ -363,11 +394,9 @@ extern "C" int llmrs_gemm(hipStream_t stream, int dtype, const void* A, int lda,
         RowScale rs{scale_sumsq, scale_parts, scale_eps};
         NextNorm nn{next_sumsq, (bf16*)next_y, next_ldy, next_weight, next_eps};
         int took = llmrs_gemm_bf16_mfma(stream, (const bf16*)A, lda, (const bf16*)W, out, ldc, M, N, K, epi, workspace,
-                                        workspace_bytes, nullptr, scale_sumsq ? &rs : nullptr, next_y ? &nn : nullptr,
-                                        epi == LLMRS_EPI_GLU_CLAMP ? &glu : nullptr);
+                                        workspace_bytes, nullptr, scale_sumsq ? &rs : nullptr, next_y ? &nn : nullptr);
         if (took != 0) return took < 0 ? -1 : 0;
     }
-    if (epi == LLMRS_EPI_GLU_CLAMP) glu_clamp_set(stream, glu);       // (this source file's kernels read their own variable)
     LLMRS_REQUIRE(scale_sumsq == nullptr && next_y == nullptr, "gemm: a deferred norm needs the bfloat16 matrix-core kernels (M=%d N=%d K=%d)", M, N, K);
     // (one or two tokens are better off with the walk below, which then asks for little beside the weights:
     // a decode step of the 8B shape at one request 7.1 against 7.8 ms)

@@ -20,7 +20,7 @@ from typing import Dict, List, NamedTuple, Optional
 import torch
 
 EPI_STORE, EPI_STORE_F32, EPI_ACCUM_F32, EPI_SWIGLU = 0, 1, 2, 3
-EPI_GLU_CLAMP = 5       # (4 is the kernel library's own: the q/k/v epilogue of `qkv_rope_cache`)
+EPI_GLU_CLAMP = 5       # and what `glu_clamp_slot` gave is added to it (4 is the kernel library's own: the q/k/v epilogue of `qkv_rope_cache`)
 _EPI_NAMES = {EPI_STORE: "store", EPI_STORE_F32: "store32", EPI_ACCUM_F32: "add32", EPI_SWIGLU: "swiglu", EPI_GLU_CLAMP: "clamped glu"}
 _EPI_GATED = (EPI_SWIGLU, EPI_GLU_CLAMP)
 
@@ -189,7 +189,8 @@ class HipKernels(Kernels):
             "llmrs_cast": [V, V, I, V, I, c_size_t],
             "llmrs_scale_softcap_rows": [V, V, I, I, I, F, F],
             "llmrs_rmsnorm": [V, I, V, V, V, V, I, I, F],
-            "llmrs_gemm": [V, I, V, I, V, V, I, I, I, I, I, V, c_size_t, I, V, I, F, V, V, I, V, F, F, F],
+            "llmrs_gemm": [V, I, V, I, V, V, I, I, I, I, I, V, c_size_t, I, V, I, F, V, V, I, V, F],
+            "llmrs_glu_clamp_slot": [V, F, F],
             "llmrs_gemm_defers_norm": [I, I, I],
             "llmrs_gemm_norms_whole": [I, I, I],
             "llmrs_gemm_next_parts": [I, I, I],
@@ -435,9 +436,10 @@ class HipKernels(Kernels):
     def gemm(self, a, w: torch.Tensor, out: torch.Tensor, epilogue: int = EPI_STORE,
              workspace: Optional[torch.Tensor] = None, leave: Optional[NextNorm] = None, glu=None) -> None:
         """`a` may be `NormedRows`, and `leave` a `NextNorm` (with the += epilogue), where `gemm_defers_norm` holds.
-        EPI_GLU_CLAMP (rows of w are gate_0, up_0, gate_1, ...; glu = (limit, alpha)): out[m, j] = g sigmoid(alpha g) (u + 1)
-        with g = min(gate_j, limit), u = clamp(up_j, -limit, limit), computed on the 32-bit sums, in the activation type."""
-        assert (glu is not None) == (epilogue == EPI_GLU_CLAMP)
+        EPI_GLU_CLAMP (rows of w are gate_0, up_0, gate_1, ...; glu = what `glu_clamp_slot(limit, alpha)` gave): out[m, j] =
+        g sigmoid(alpha g) (u + 1) with g = min(gate_j, limit), u = clamp(up_j, -limit, limit), computed on the 32-bit sums,
+        in the activation type."""
+        assert (glu is not None) == (epilogue == EPI_GLU_CLAMP) and (glu is None or isinstance(glu, int))
         scale = None
         if isinstance(a, NormedRows):
             scale, a = a, a.y
@@ -462,13 +464,21 @@ class HipKernels(Kernels):
         label = f"gemm {M}x{N}x{K} {'norm+' if scale is not None else ''}{_EPI_NAMES[epilogue]}{('+norm' if whole else '+next') if leave is not None else ''}"
         self._run(label, moved, 2 * M * N * K, a.dtype,
                   self.lib.llmrs_gemm, self._stream(), _code(a.dtype), _p(a), a.stride(0), _p(w), _p(out), out.stride(0),
-                  M, N, K, epilogue, _p(workspace),
+                  M, N, K, epilogue + (glu or 0), _p(workspace),
                   0 if workspace is None else workspace.numel() * workspace.element_size(), int(self.allow_mfma),
                   None if scale is None else _p(scale.sumsq), 0 if scale is None else scale.sumsq.shape[1],
                   0.0 if scale is None else scale.eps, None if leave is None or whole else _p(leave.sumsq),
                   None if leave is None else _p(leave.y), 0 if leave is None else leave.y.stride(0),
-                  None if leave is None else _p(leave.weight), leave.eps if whole else 0.0,
-                  0.0 if glu is None else float(glu[0]), 0.0 if glu is None else float(glu[1]))
+                  None if leave is None else _p(leave.weight), leave.eps if whole else 0.0)
+
+    def glu_clamp_slot(self, limit: float, alpha: float) -> int:
+        """Where the kernel library keeps this pair of constants of the clamped gated epilogue on the current device: what
+        `gemm(..., EPI_GLU_CLAMP, glu=...)` takes.  Asked for when a feed-forward takes its weights, never inside a
+        recording (the first call for a pair writes device memory and waits for the stream)."""
+        slot = int(self.lib.llmrs_glu_clamp_slot(self._stream(), float(limit), float(alpha)))
+        if slot < 0:
+            raise KernelError(self.lib.llmrs_hip_error().decode())
+        return slot
 
     def rope_kv_write(self, qkv, positions, slot_map, inv_freq, rotary_dim, interleaved, k_cache, v_cache,
                       n_heads, n_kv_heads, head_dim, page_size, num_pages, write_kv) -> None:
@@ -932,6 +942,11 @@ def kernels():
     if _kernels is None:
         _kernels = HipKernels()
     return _kernels
+
+
+def stand_in_kernels() -> bool:
+    """Whether another object stands in for the kernel library (`use_kernels`: tests of the host logic without a GPU)."""
+    return _kernels is not None and not isinstance(_kernels, HipKernels)
 
 
 @contextlib.contextmanager

@@ -6,9 +6,11 @@ side and its epilogue writes silu(gate) * up, computed in 32-bit, once; the down
 product adds into the 32-bit residual stream.  No biases."""
 from __future__ import annotations
 
+import contextlib
+
 import torch
 
-from ..kernels import EPI_ACCUM_F32, EPI_GLU_CLAMP, EPI_STORE_F32, EPI_SWIGLU, kernels
+from ..kernels import EPI_ACCUM_F32, EPI_GLU_CLAMP, EPI_STORE_F32, EPI_SWIGLU, kernels, stand_in_kernels
 from .base import FeedForward, TensorSpec, build_feed_forward, place, register_feed_forward
 
 
@@ -77,7 +79,7 @@ class ClampedGLU(FeedForward):
             raise ValueError(f"the activation's limit must be positive, got {self.limit}")
         leaves = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight", **(p.get("names") or {})}
         self.n_gate, self.n_up, self.n_down = (self.name(leaves[k]) for k in ("gate", "up", "down"))
-        self.w_gate_up = self.w_down = None
+        self.w_gate_up = self.w_down = self.glu = None
 
     def tensors(self):
         return {self.n_gate: TensorSpec((self.inter, self.hidden)), self.n_up: TensorSpec((self.inter, self.hidden)),
@@ -87,6 +89,11 @@ class ClampedGLU(FeedForward):
         gate, up = place(tensors[self.n_gate], device, self.dtype), place(tensors[self.n_up], device, self.dtype)
         self.w_gate_up = torch.stack([gate, up], dim=1).reshape(2 * self.inter, self.hidden).contiguous()
         self.w_down = place(tensors[self.n_down], device, self.dtype)
+        # where the kernels keep the activation's two constants (asked for here, outside any recording)
+        # (a model on the CPU with no stand-in for the kernels only holds its weights)
+        on_device = torch.device(device).type == "cuda"
+        with torch.cuda.device(device) if on_device else contextlib.nullcontext():
+            self.glu = kernels().glu_clamp_slot(self.limit, self.alpha) if on_device or stand_in_kernels() else None
 
     def export(self):
         both = self.w_gate_up.cpu().view(self.inter, 2, self.hidden)
@@ -96,7 +103,7 @@ class ClampedGLU(FeedForward):
         k = kernels()
         T = x.shape[0]
         act = ctx.workspace("mlp.act", (T, self.inter), self.dtype)
-        k.gemm(x, self.w_gate_up, act, EPI_GLU_CLAMP, ctx.gemm_workspace(x, self.w_gate_up), glu=(self.limit, self.alpha))
+        k.gemm(x, self.w_gate_up, act, EPI_GLU_CLAMP, ctx.gemm_workspace(x, self.w_gate_up), glu=self.glu)
         k.gemm(act, self.w_down, h, EPI_ACCUM_F32, ctx.gemm_workspace(act, self.w_down))
         ctx.note_left(h, None)
 

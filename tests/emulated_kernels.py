@@ -119,6 +119,9 @@ class EmulatedKernels(Kernels):
     def norm_left_by_product(self, M, N, K, dtype):
         return NormPlan(False, -(-N // 16)) if dtype == torch.bfloat16 and 1 <= M <= 16 else None
 
+    def glu_clamp_slot(self, limit, alpha):
+        return (float(limit), float(alpha))          # (no table here: the constants themselves are what gemm is given)
+
     def gemm(self, a, w, out, epilogue=EPI_STORE, workspace=None, leave=None, glu=None):
         inv = None
         if hasattr(a, "sumsq"):        # kernels.NormedRows: rows times the norm's weight, rounded; the scale comes after the sums

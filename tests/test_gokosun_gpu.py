@@ -151,7 +151,8 @@ def test_the_router_with_sigmoid_scores_and_a_correction(E, top):
 @pytest.mark.parametrize("N,K", [(14, 10), (64, 64), (512, 320), (2048, 256), (6144, 1024)])
 def test_the_gate_and_up_product_with_the_clamped_activation(M, N, K, dtype):
     """Every tiling of the product (by its number of rows and its widths) finishes the same activation; two different
-    limits one after the other, as two feed-forwards of a layer have them."""
+    pairs of constants one after the other, as two feed-forwards of a layer have them, each in a slot of its own that
+    the same pair gets again."""
     from llm_rs_amd.kernels import EPI_GLU_CLAMP
     x, w = (rand(M, K, seed=M) * 0.8).to(dtype), (rand(N, K, seed=N) * 0.2).to(dtype)
     sums = x.double() @ w.double().T
@@ -162,8 +163,9 @@ def test_the_gate_and_up_product_with_the_clamped_activation(M, N, K, dtype):
         k = kernels()
         n_ws = k.gemm_workspace_floats(M, N, K)
         ws = torch.empty(n_ws, device="cuda") if n_ws else None
-        k.gemm(x.cuda(), w.cuda(), out, EPI_GLU_CLAMP, ws, glu=(limit, alpha))
+        k.gemm(x.cuda(), w.cuda(), out, EPI_GLU_CLAMP, ws, glu=k.glu_clamp_slot(limit, alpha))
         close(out, want, dtype, f"limit {limit}", tol=5e-5 if dtype == torch.float32 else 1e-2)
+        assert k.glu_clamp_slot(limit, alpha) == k.glu_clamp_slot(limit, alpha) != k.glu_clamp_slot(limit + 1.0, alpha)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
