@@ -20,7 +20,7 @@ enum LlmrsEpilogue {
 // model has (llmrs_glu_clamp_slot, called when a feed-forward takes its weights, writes a slot once and for all); the
 // epilogue's number says which slot, so no kernel's argument list holds them and a recorded step finds them as any
 // other does.  Each source file with such kernels has the table for itself (the variable is static).
-#define LLMRS_GLU_SLOTS 64
+#define LLMRS_GLU_SLOTS 256
 struct GluClamp {
     float limit, alpha;
 };

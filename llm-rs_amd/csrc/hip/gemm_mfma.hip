@@ -53,13 +53,26 @@ __device__ __forceinline__ float swap_neighbours(float x) {
 __device__ __forceinline__ float silu_fast_f32(float x) {
     return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * -1.44269504088896341f));
 }
-// act(gate, up) of the two gated epilogues with the same instructions
-__device__ __forceinline__ float gated_act_fast(int epi, float g, float u) {
-    if (epi == LLMRS_EPI_SWIGLU) return silu_fast_f32(g) * u;
-    const GluClamp p = llmrs_glu_clamp[epi - LLMRS_EPI_GLU_CLAMP];
-    g = fminf(g, p.limit);
-    u = fminf(fmaxf(u, -p.limit), p.limit);
-    return g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g * (p.alpha * -1.44269504088896341f))) * (u + 1.0f);
+// act(gate, up) of the gated epilogues with the same instructions; the clamped one's constants are read from their slot
+// once, before the loops that finish a tile (gated_act_of), not value by value
+struct GatedAct {
+    int epi;
+    float limit, alpha2;        // alpha2 = -alpha log2(e)
+};
+__device__ __forceinline__ GatedAct gated_act_of(int epi) {
+    GatedAct a{epi, 0.0f, 0.0f};
+    if (epi >= LLMRS_EPI_GLU_CLAMP) {
+        const GluClamp p = llmrs_glu_clamp[epi - LLMRS_EPI_GLU_CLAMP];
+        a.limit = p.limit;
+        a.alpha2 = p.alpha * -1.44269504088896341f;
+    }
+    return a;
+}
+__device__ __forceinline__ float gated_act_fast(const GatedAct& a, float g, float u) {
+    if (a.epi == LLMRS_EPI_SWIGLU) return silu_fast_f32(g) * u;
+    g = fminf(g, a.limit);
+    u = fminf(fmaxf(u, -a.limit), a.limit);
+    return g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g * a.alpha2)) * (u + 1.0f);
 }
 void llmrs_glu_clamp_store_mfma(hipStream_t stream, int slot, GluClamp p) { glu_clamp_store_kernel<<<1, 1, 0, stream>>>(slot, p); }
 
@@ -620,6 +633,7 @@ __device__ __forceinline__ void tile_epilogue(f32x16 (&acc)[BM / WGM / 32][BN / 
                   (epi_gated(epi) ? N % 16 == 0 : N % 8 == 0);
     if (staged) {
         const bool glu = epi_gated(epi);
+        const GatedAct ga = gated_act_of(epi);
         const int cols = glu ? TN / 2 : TN;                       // columns of the wave's tile as stored
         const int row_bytes = cols * 2;
         static_assert(TN * 2 * TM * WAVES <= SMEM_BYTES, "the waves' tiles must fit in the tile buffers");
@@ -639,7 +653,7 @@ __device__ __forceinline__ void tile_epilogue(f32x16 (&acc)[BM / WGM / 32][BN / 
                 float v0 = acc[i][j][r], v1 = acc[i][j][r + 1];
                 float got = swap_neighbours(odd ? v0 : v1);
                 float left = odd ? got : v0, right = odd ? v1 : got;       // columns c & ~1 and c | 1 of `row`
-                if (glu) *(bf16*)(mine + row * row_bytes + (c / 2) * 2) = (bf16)gated_act_fast(epi, left, right);
+                if (glu) *(bf16*)(mine + row * row_bytes + (c / 2) * 2) = (bf16)gated_act_fast(ga, left, right);
                 else {
                     bf16x2 two;
                     two[0] = (bf16)left;
@@ -1036,6 +1050,7 @@ __device__ __forceinline__ void band_epilogue(f32x16 (&acc)[BM / 64][BN / 64], u
         });
     } else {
         constexpr bool glu = EPI == LLMRS_EPI_SWIGLU || EPI == LLMRS_EPI_GLU_CLAMP;
+        const GatedAct ga = gated_act_of(EPI == LLMRS_EPI_GLU_CLAMP ? epi : EPI);
         constexpr int cols = glu ? TN / 2 : TN;      // columns of the wave's band as stored
         constexpr int row_bytes = cols * 2;
         unsigned char* mine = smem + wave * (32 * TN * 2);
@@ -1053,7 +1068,7 @@ __device__ __forceinline__ void band_epilogue(f32x16 (&acc)[BM / 64][BN / 64], u
                     float v0 = acc[i][j][r], v1 = acc[i][j][r + 1];
                     float got = swap_neighbours(odd ? v0 : v1);
                     float left = odd ? got : v0, right = odd ? v1 : got;
-                    if (glu) *(bf16*)(mine + row * row_bytes + (cc / 2) * 2) = (bf16)gated_act_fast(EPI == LLMRS_EPI_GLU_CLAMP ? epi : EPI, left, right);
+                    if (glu) *(bf16*)(mine + row * row_bytes + (cc / 2) * 2) = (bf16)gated_act_fast(ga, left, right);
                     else {
                         bf16x2 two;
                         two[0] = (bf16)left;

@@ -10,7 +10,7 @@ import contextlib
 
 import torch
 
-from ..kernels import EPI_ACCUM_F32, EPI_GLU_CLAMP, EPI_STORE_F32, EPI_SWIGLU, kernels, stand_in_kernels
+from ..kernels import EPI_ACCUM_F32, EPI_GLU_CLAMP, EPI_STORE_F32, EPI_SWIGLU, KernelError, kernels, stand_in_kernels
 from .base import FeedForward, TensorSpec, build_feed_forward, place, register_feed_forward
 
 
@@ -93,7 +93,10 @@ class ClampedGLU(FeedForward):
         # (a model on the CPU with no stand-in for the kernels only holds its weights)
         on_device = torch.device(device).type == "cuda"
         with torch.cuda.device(device) if on_device else contextlib.nullcontext():
-            self.glu = kernels().glu_clamp_slot(self.limit, self.alpha) if on_device or stand_in_kernels() else None
+            try:
+                self.glu = kernels().glu_clamp_slot(self.limit, self.alpha) if on_device or stand_in_kernels() else None
+            except KernelError:         # (every slot taken: the activation then runs as a kernel of its own on the 32-bit sums)
+                self.glu = None
 
     def export(self):
         both = self.w_gate_up.cpu().view(self.inter, 2, self.hidden)
@@ -103,7 +106,12 @@ class ClampedGLU(FeedForward):
         k = kernels()
         T = x.shape[0]
         act = ctx.workspace("mlp.act", (T, self.inter), self.dtype)
-        k.gemm(x, self.w_gate_up, act, EPI_GLU_CLAMP, ctx.gemm_workspace(x, self.w_gate_up), glu=self.glu)
+        if self.glu is not None:
+            k.gemm(x, self.w_gate_up, act, EPI_GLU_CLAMP, ctx.gemm_workspace(x, self.w_gate_up), glu=self.glu)
+        else:
+            sums = ctx.workspace("mlp.up", (T, 2 * self.inter), torch.float32)
+            k.gemm(x, self.w_gate_up, sums, EPI_STORE_F32, ctx.gemm_workspace(x, self.w_gate_up))
+            k.act_weight(act, sums, None, self.inter, "clamped_glu", self.limit, self.alpha)
         k.gemm(act, self.w_down, h, EPI_ACCUM_F32, ctx.gemm_workspace(act, self.w_down))
         ctx.note_left(h, None)
 
